@@ -787,6 +787,70 @@ int mi355_moe_grouped_linear(void* out, const void* in, int64_t in_stride, const
                              const int32_t* tile_expert, const int32_t* n_tiles, int gather, int gelu, int64_t padded, int block,
                              int n, int k, int dtype, void* stream);
 
+/* mi355_moe_route_scores: the same selection with its choices spelled out: score_fn 0 = sigmoid, 1 = softmax over all
+ *   experts; correction may be null; a group scores the sum of its group_best (1 or 2) largest selection scores;
+ *   renorm 0 leaves the weights at s[chosen] * scale. */
+int mi355_moe_route_scores(int32_t* ids, float* weights, const float* logits, const float* correction, int64_t tokens,
+                           int num_experts, int top, int n_groups, int keep_groups, float scale, int score_fn, int group_best,
+                           int renorm, void* stream);
+
+/* ---- pre-norm 32-bit stream with parallel branches ------------------------------------------------------
+ * mi355_offset_rmsnorm: h[t] = x[t] / sqrt(mean(x[t]^2) + eps) * (offset + weight), x fp32, h and weight of type T.
+ * mi355_branch_residual_add: x[t] += s * (A + B) + F in place on the fp32 rows; A = a[t] / sqrt(mean(a[t]^2) + eps) * wa
+ *   (wa null: a[t] as it is), B the same from b, wb (b null: none), F = f[t] (rows null), or the sum over j < n_branch of
+ *   coef[t][j] * f[rows[t][j]] in that order, or nothing (f null).
+ * mi355_head_rmsnorm_gate_act: mi355_head_rmsnorm_gate with the gate's function chosen: 0 = silu, 1 = sigmoid. */
+int mi355_offset_rmsnorm(void* h, const float* x, const void* weight, int64_t tokens, int64_t hidden, float eps, float offset,
+                         int dtype, void* stream);
+int mi355_branch_residual_add(float* x, const void* a, int64_t a_stride, const void* wa, const void* b, int64_t b_stride,
+                              const void* wb, float s, const void* f, int64_t f_stride, const int32_t* rows, const float* coef,
+                              int n_branch, int64_t tokens, int64_t hidden, float eps, int dtype, void* stream);
+int mi355_head_rmsnorm_gate_act(void* out, const float* o, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,
+                                int heads, int value_dim, float eps, int gate_act, int dtype, void* stream);
+
+/* ---- short causal convolutions over time with per-sequence state ----------------------------------------
+ * mi355_causal_conv: y[t][c] = act((residual ? u[t][c] : 0) + sum_{k < taps} w[c][taps - 1 - k] * u_(t - k)[c]); u_(t - k) is
+ *   the step's own row while it belongs to the same sequence (tok_req / seg_start; both null: every token is a sequence of
+ *   its own), else state[slot][taps - 1 - (k - back)][c] (fp32 [slots, taps - 1, channels], `back` = tokens of the step
+ *   before t in its sequence), else 0 (before position 0).  w2 / y2: a second filter over the same input (null: none).
+ *   act 0 none, 1 silu, 2 squared relu.  Without segments the launch also shifts the state; with segments
+ *   mi355_causal_conv_state_update does, afterwards: the last taps - 1 of (old rows, the step's inputs).
+ * mi355_activation: out[r][i] = act(in[r * in_stride + i]), act 1 or 2 as above. */
+int mi355_causal_conv(void* y1, void* y2, const void* u, int64_t u_stride, const void* w1, const void* w2, float* state,
+                      const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* tok_req,
+                      const int32_t* seg_start, const int64_t* positions, int64_t tokens, int64_t channels, int taps,
+                      int residual, int act, int dtype, void* stream);
+int mi355_causal_conv_state_update(float* state, const void* u, int64_t u_stride, const int32_t* req_to_state,
+                                   const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                                   const int64_t* positions, int64_t batch, int64_t channels, int taps, int dtype, void* stream);
+int mi355_activation(void* out, const void* in, int64_t in_stride, int64_t rows, int64_t cols, int act, int dtype, void* stream);
+
+/* ---- gated delta rule with one fp32 matrix per (sequence, head) --------------------------------------
+ * As mi355_linear_recurrence, with per token  S = diag(a) S;  u = beta (v - S^T k);  S = S + k u^T;  out = S^T (q * q_scale);
+ *   a[i] = exp(-exp(rate_log[h]) * softplus(gate_logits[t][h * key_dim + i] + rate_bias[h * key_dim + i])) (all fp32),
+ *   beta = sigmoid(beta_logits[t * beta_token_stride + h]) (v's type).  q, k [tokens, qk_heads, key_dim]: head h reads
+ *   q / k head h / (heads / qk_heads). */
+int mi355_gated_delta_rule(float* out, float* state, const void* q, const void* k, const void* v, const void* beta_logits,
+                           const float* gate_logits, const float* rate_bias, const float* rate_log, const int32_t* req_to_state,
+                           const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                           const int64_t* positions, int64_t batch, int heads, int qk_heads, int key_dim, int value_dim,
+                           int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, int64_t beta_token_stride,
+                           int64_t gate_token_stride, float q_scale, int qk_dtype, int v_dtype, void* stream);
+
+/* ---- softmax attention over a sliding window with a sink in the denominator -----------------------------
+ * out[t][h] = sum_j exp(s_j) V[j][g] / (exp(sink[h]) + sum_j exp(s_j)), s_j = (q[t][h] . K[j][g]) * scale over the keys j of
+ *   t's sequence with 0 <= pos(t) - j < window (window <= 0: all j <= pos(t)), g = h / (heads / kv_heads); sink null: no
+ *   such term.  Caches [slots, kv_heads, head_dim] / [slots, kv_heads, v_head_dim] reached through req_to_token; `blocks`
+ *   int32 [num_blocks][2] runs (first token, count <= block_tokens) of consecutive tokens of one sequence, or null (one
+ *   token per run); max_run: the longest run.  The new tokens' keys and values must be in the caches already. */
+int mi355_window_attention_block_tokens(int heads, int kv_heads, int head_dim, int v_head_dim, int dtype);
+int mi355_window_attention(void* out, const void* q, const void* k_cache, const void* v_cache, const int32_t* req_to_token,
+                           const int64_t* req_pool_indices, const int32_t* tok_req, const int64_t* positions,
+                           const int32_t* blocks, int64_t num_blocks, const float* sink, int64_t q_token_stride,
+                           int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t req_to_token_stride,
+                           int heads, int kv_heads, int head_dim, int v_head_dim, int window, float scale, int64_t tokens,
+                           int max_run, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

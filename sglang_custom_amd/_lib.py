@@ -117,6 +117,16 @@ _SIGNATURES = {
     "mi355_moe_router_logits": (I, [P, P, P, L, I, I, P]),
     "mi355_moe_align": (I, [P, P, P, P, P, L, I, I, I, L, P]),
     "mi355_moe_grouped_linear": (I, [P, P, L, P, P, P, P, I, I, L, I, I, I, I, P]),
+    "mi355_moe_route_scores": (I, [P, P, P, P, L, I, I, I, I, F, I, I, I, P]),
+    "mi355_offset_rmsnorm": (I, [P, P, P, L, L, F, F, I, P]),
+    "mi355_branch_residual_add": (I, [P, P, L, P, P, L, P, F, P, L, P, P, I, L, L, F, I, P]),
+    "mi355_head_rmsnorm_gate_act": (I, [P, P, P, P, L, L, I, I, F, I, I, P]),
+    "mi355_causal_conv": (I, [P, P, P, L, P, P, P, P, P, P, P, P, L, L, I, I, I, I, P]),
+    "mi355_causal_conv_state_update": (I, [P, P, L, P, P, P, P, P, L, L, I, I, P]),
+    "mi355_activation": (I, [P, P, L, L, L, I, I, P]),
+    "mi355_gated_delta_rule": (I, [P, P, P, P, P, P, P, P, P, P, P, P, P, P, L, I, I, I, I, L, L, L, L, L, F, I, I, P]),
+    "mi355_window_attention_block_tokens": (I, [I, I, I, I, I]),
+    "mi355_window_attention": (I, [P, P, P, P, P, P, P, P, P, L, P, L, L, L, L, L, I, I, I, I, I, F, L, I, I, P]),
     "mi355_latent_window_attention": (I, [P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, L, L, I, I, I, I, I, F, I, P, L, I, P]),
 }
 

@@ -14,7 +14,7 @@ LIB = os.path.join(HERE, "libmi355_hotpath.so")
 LIB_DEV = os.path.join(HERE, "libmi355_hotpath_dev.so")
 SOURCES = ["elementwise.hip", "index_ops.hip", "attn_decode.hip", "attn_extend.hip", "gemm.hip",
            "gemm_tiled.hip", "sampling.hip", "quant_fp8.hip", "allreduce.hip", "mla_proj.hip",
-           "stream_ops.hip", "attn_latent.hip", "postnorm_ops.hip", "recurrence.hip", "attn_sigmoid.hip", "moe_ops.hip"]
+           "stream_ops.hip", "attn_latent.hip", "postnorm_ops.hip", "recurrence.hip", "attn_sigmoid.hip", "moe_ops.hip", "conv_ops.hip", "attn_window.hip"]
 DEV_SOURCES = ["debug_bw.hip"]
 HEADERS = [os.path.join(CSRC, "common.cuh"),
            os.path.join(os.path.dirname(HERE), "include", "mi355_hotpath.h"),
@@ -44,6 +44,8 @@ FAMILY_SOURCES = {
     "Seturax": ["elementwise.hip", "index_ops.hip", "gemm.hip", "gemm_tiled.hip", "stream_ops.hip", "attn_latent.hip"],
     "Verozen": ["elementwise.hip", "index_ops.hip", "gemm.hip", "gemm_tiled.hip", "postnorm_ops.hip", "recurrence.hip",
                 "attn_sigmoid.hip", "moe_ops.hip"],
+    "Gatarax": ["elementwise.hip", "index_ops.hip", "gemm.hip", "gemm_tiled.hip", "postnorm_ops.hip", "recurrence.hip",
+                "moe_ops.hip", "conv_ops.hip", "attn_window.hip"],
 }
 PARTIAL_MARK = LIB + ".partial"
 

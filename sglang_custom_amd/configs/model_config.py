@@ -26,6 +26,9 @@ class ModelConfig:
         if self.architecture == "Verozen":
             self._init_verozen(c, dtype, context_length, quantization)
             return
+        if self.architecture == "Gatarax":
+            self._init_gatarax(c, dtype, context_length, quantization)
+            return
         self.hidden_size = c["hidden_size"]
         self.num_hidden_layers = c["num_hidden_layers"]
         self.num_attention_heads = c["num_attention_heads"]
@@ -146,6 +149,59 @@ class ModelConfig:
         # per layer (heads, key width, value width) of the state matrices of the recurrent layers, None for the others
         self.recurrent_layer_shapes = [(s["mixer"]["heads"], s["mixer"]["dim"], s["mixer"]["vdim"])
                                        if s["type"] != "attention" else None for s in layers]
+
+    def _init_gatarax(self, c: dict, dtype: str, context_length: Optional[int], quantization: Optional[str]) -> None:
+        """The Gatarax design: "layers" lists the layers one by one, {"type": "parallel" | "lightning", "mixer": {...},
+        "mlp": {"kind": "dense", "ff"} | {"kind": "moe", "expert": {"ff"}, "router": {...}} | null}; widths under "width" /
+        "vocab", the norms' epsilon under "norm", the embedding's factor under "embedding", the taps of the convolution in
+        front of every sublayer under "canon", the factor of the logits under "logit_scale".  A "parallel" mixer holds a
+        windowed attention branch ("left": keys and values per token, kv_layer_shapes) beside a gated-delta-rule branch
+        ("right": one matrix per head and sequence); a "lightning" mixer is a linear recurrence with a fixed decay per
+        head.  Layers may differ in every size."""
+        layers = c["layers"]
+        for i, spec in enumerate(layers):
+            if spec["type"] not in ("parallel", "lightning"):
+                raise ValueError(f"Gatarax layer {i}: unknown mixer type {spec['type']!r}")
+            if spec.get("mlp") is not None and spec["mlp"].get("kind") not in ("dense", "moe"):
+                raise ValueError(f"Gatarax layer {i}: unknown feed-forward kind {spec['mlp'].get('kind')!r}")
+            m = spec["mixer"]
+            if spec["type"] == "parallel":
+                for side in ("left", "right"):
+                    b = m[side]
+                    if b["heads"] % b.get("kv_heads", b["heads"]):
+                        raise ValueError(f"Gatarax layer {i} {side}: {b['heads']} heads over {b['kv_heads']} key heads")
+            elif len(m["decay"]) != m["heads"]:
+                raise ValueError(f"Gatarax layer {i}: {len(m['decay'])} decays for {m['heads']} heads")
+        self.layer_specs = layers
+        self.hidden_size = c["width"]
+        self.vocab_size = c["vocab"]
+        self.num_hidden_layers = len(layers)
+        att = [s["mixer"]["left"] for s in layers if s["type"] == "parallel"]
+        self.num_attention_heads = max([m["heads"] for m in att] or [1])
+        self.num_key_value_heads = max([m.get("kv_heads", m["heads"]) for m in att] or [1])
+        self.head_dim = max([m["dim"] for m in att] or [1])
+        self.v_head_dim = max([m.get("vdim", m["dim"]) for m in att] or [1])
+        self.intermediate_size = max([s["mlp"]["ff"] if s["mlp"]["kind"] == "dense" else s["mlp"]["expert"]["ff"]
+                                      for s in layers if s.get("mlp")] or [0])
+        self.rms_norm_eps = c["norm"]["eps"]
+        self.embedding_scale = float((c.get("embedding") or {}).get("scale", 1.0))
+        self.canon_taps = int((c.get("canon") or {}).get("taps", 0))
+        self.logit_scale = float(c.get("logit_scale", 1.0))
+        self.rope_theta = None
+        self.rope_scaling = None
+        self.tie_word_embeddings = True
+        self.max_position_embeddings = context_length or 131072     # the design fixes no longest sequence
+        self.context_len = self.max_position_embeddings
+        self.quantization = quantization
+        self.dtype = _DTYPES.get(dtype) or torch.bfloat16
+        self.is_encoder_decoder = False
+        self.needs_sequence_state = True      # convolution inputs and recurrent matrices travel from step to step
+        self.kv_layer_shapes = [(s["mixer"]["left"].get("kv_heads", s["mixer"]["left"]["heads"]), s["mixer"]["left"]["dim"],
+                                 s["mixer"]["left"].get("vdim", s["mixer"]["left"]["dim"]))
+                                if s["type"] == "parallel" else None for s in layers]
+        self.recurrent_layer_shapes = [(s["mixer"]["right"]["heads"], s["mixer"]["right"]["dim"], s["mixer"]["right"]["vdim"])
+                                       if s["type"] == "parallel" else (s["mixer"]["heads"], s["mixer"]["dim"], s["mixer"]["vdim"])
+                                       for s in layers]
 
     @classmethod
     def from_path(cls, model_path: str, **kw) -> "ModelConfig":

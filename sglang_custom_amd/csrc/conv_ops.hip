@@ -1,0 +1,162 @@
+// Short causal convolutions over time, one filter per channel, for sequences that arrive in pieces:
+//     y[t][c] = act( (residual ? u[t][c] : 0) + sum_{k < taps} w[c][taps - 1 - k] * u[t - k][c] ),   u = 0 before position 0
+// The last taps - 1 inputs of a sequence are its state (fp32 rows [slots, taps - 1, C], row taps - 2 the most recent): a
+// step's first tokens read them, and after the step they are replaced by the step's own last inputs.
+//   * mi355_causal_conv: every (token, channel) in one launch; up to two filters read the same input (two outputs).  In a
+//     step of single tokens (no segments) the same thread also shifts the state, so decode is one launch.
+//   * mi355_causal_conv_state_update: the shift for steps with segments, one thread per (sequence, channel), after the
+//     convolution has read the old rows.
+//   * mi355_activation: out = act(in) over a strided [rows, cols] block (silu, squared relu).
+// The sum runs over the taps in a fixed order in fp32 whether an input comes from the step or from the state, so a
+// position's result does not depend on how its sequence was cut.
+#include "common.cuh"
+
+#include <algorithm>
+
+namespace mi355 {
+namespace {
+
+constexpr int CONV_MAX_TAPS = 8;
+
+__device__ __forceinline__ float conv_act(float z, int act) {
+  if (act == 1) return z / (1.0f + expf(-z));
+  if (act == 2) { const float r = fmaxf(z, 0.f); return r * r; }
+  return z;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_kernel(T* __restrict__ y1, T* __restrict__ y2, const T* __restrict__ u,
+                                                          int64_t u_stride, const T* __restrict__ w1, const T* __restrict__ w2,
+                                                          float* __restrict__ state, const int32_t* __restrict__ req_to_state,
+                                                          const int64_t* __restrict__ req_pool_indices,
+                                                          const int32_t* __restrict__ tok_req, const int32_t* __restrict__ seg_start,
+                                                          const int64_t* __restrict__ positions, int64_t C, int taps, int residual,
+                                                          int act) {
+  const int64_t t = blockIdx.x;
+  const int64_t c = (int64_t)blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int b = tok_req != nullptr ? tok_req[t] : (int)t;
+  const int64_t t0 = seg_start != nullptr ? seg_start[b] : t;
+  const int64_t pos = positions[t];
+  const int back = (int)(t - t0);                 // tokens of this step before t in its sequence
+  float* rows = state + (int64_t)req_to_state[req_pool_indices[b]] * (taps - 1) * C + c;
+  float in[CONV_MAX_TAPS];                         // in[k]: the input k tokens back
+#pragma unroll
+  for (int k = 0; k < CONV_MAX_TAPS; ++k) {
+    if (k >= taps) break;
+    float v = 0.f;
+    if (k <= back) v = to_f32(u[(t - k) * u_stride + c]);
+    else if (pos - k >= 0) v = rows[(int64_t)(taps - 1 - (k - back)) * C];
+    in[k] = v;
+  }
+  float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+  for (int k = CONV_MAX_TAPS - 1; k >= 0; --k) {   // oldest tap first
+    if (k >= taps) continue;
+    a1 = fmaf(to_f32(w1[c * taps + (taps - 1 - k)]), in[k], a1);
+    if (w2 != nullptr) a2 = fmaf(to_f32(w2[c * taps + (taps - 1 - k)]), in[k], a2);
+  }
+  if (residual) { a1 += in[0]; a2 += in[0]; }
+  y1[t * C + c] = from_f32<T>(conv_act(a1, act));
+  if (w2 != nullptr) y2[t * C + c] = from_f32<T>(conv_act(a2, act));
+  if (tok_req == nullptr) {
+    // a step of single tokens: this thread is the only reader and writer of its channel's rows
+#pragma unroll
+    for (int k = CONV_MAX_TAPS - 2; k >= 0; --k) {
+      if (k >= taps - 1) continue;
+      rows[(int64_t)(taps - 2 - k) * C] = in[k];
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_state_update_kernel(float* __restrict__ state, const T* __restrict__ u,
+                                                                       int64_t u_stride, const int32_t* __restrict__ req_to_state,
+                                                                       const int64_t* __restrict__ req_pool_indices,
+                                                                       const int32_t* __restrict__ seg_start,
+                                                                       const int32_t* __restrict__ seg_len,
+                                                                       const int64_t* __restrict__ positions, int64_t C, int taps) {
+  const int b = blockIdx.y;
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int n = seg_len[b];
+  if (n <= 0) return;
+  const int64_t t0 = seg_start[b];
+  const int64_t p0 = positions[t0];
+  float* rows = state + (int64_t)req_to_state[req_pool_indices[b]] * (taps - 1) * C + c;
+  // the old rows followed by the step's inputs; the new rows are the last taps - 1 of that list.  Row i takes entry
+  // n + i >= i + 1, so going up never reads a row already replaced.
+  for (int i = 0; i < taps - 1; ++i) {
+    const int e = n + i;
+    float v;
+    if (e < taps - 1) v = (p0 - (taps - 1) + e >= 0) ? rows[(int64_t)e * C] : 0.f;
+    else v = to_f32(u[(t0 + e - (taps - 1)) * u_stride + c]);
+    rows[(int64_t)i * C] = v;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ out, const T* __restrict__ in, int64_t in_stride,
+                                                         int64_t rows, int64_t cols, int act) {
+  const int64_t n = rows * cols;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = idx / cols, i = idx - r * cols;
+    out[idx] = from_f32<T>(conv_act(to_f32(in[r * in_stride + i]), act));
+  }
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+int mi355_causal_conv(void* y1, void* y2, const void* u, int64_t u_stride, const void* w1, const void* w2, float* state,
+                      const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* tok_req,
+                      const int32_t* seg_start, const int64_t* positions, int64_t tokens, int64_t channels, int taps,
+                      int residual, int act, int dtype, void* stream) {
+  MI355_REQUIRE(y1 && u && w1 && (state || taps == 1) && req_to_state && req_pool_indices && positions, MI355_ERR_INVALID, "causal_conv: null pointer");
+  MI355_REQUIRE((w2 == nullptr) == (y2 == nullptr), MI355_ERR_INVALID, "causal_conv: the second filter comes with its output");
+  MI355_REQUIRE((tok_req == nullptr) == (seg_start == nullptr), MI355_ERR_INVALID, "causal_conv: tok_req and seg_start come together");
+  MI355_REQUIRE(tokens >= 0 && tokens <= 0x7fffffff && channels > 0 && u_stride >= channels && taps >= 1 && taps <= CONV_MAX_TAPS &&
+                    act >= 0 && act <= 2, MI355_ERR_INVALID, "causal_conv: bad shape (1 to %d taps)", CONV_MAX_TAPS);
+  if (tokens == 0) return MI355_OK;
+  MI355_REQUIRE(channels <= 65535 * 256, MI355_ERR_UNSUPPORTED, "causal_conv: too many channels");
+  const dim3 grid((unsigned)tokens, (unsigned)cdiv(channels, 256));
+  MI355_DISPATCH_DTYPE(dtype, "causal_conv", {
+    hipLaunchKernelGGL((causal_conv_kernel<T>), grid, dim3(256), 0, (hipStream_t)stream, (T*)y1, (T*)y2, (const T*)u, u_stride,
+                       (const T*)w1, (const T*)w2, state, req_to_state, req_pool_indices, tok_req, seg_start, positions, channels,
+                       taps, residual, act);
+  });
+  MI355_CHECK_LAUNCH("causal_conv");
+  return MI355_OK;
+}
+
+int mi355_causal_conv_state_update(float* state, const void* u, int64_t u_stride, const int32_t* req_to_state,
+                                   const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                                   const int64_t* positions, int64_t batch, int64_t channels, int taps, int dtype, void* stream) {
+  MI355_REQUIRE((state || taps == 1) && u && req_to_state && req_pool_indices && seg_start && seg_len && positions, MI355_ERR_INVALID,
+                "causal_conv_state_update: null pointer");
+  MI355_REQUIRE(batch >= 0 && batch <= 65535 && channels > 0 && u_stride >= channels && taps >= 1 && taps <= CONV_MAX_TAPS,
+                MI355_ERR_INVALID, "causal_conv_state_update: bad shape");
+  if (batch == 0 || taps == 1) return MI355_OK;
+  const dim3 grid((unsigned)cdiv(channels, 256), (unsigned)batch);
+  MI355_DISPATCH_DTYPE(dtype, "causal_conv_state_update", {
+    hipLaunchKernelGGL((causal_conv_state_update_kernel<T>), grid, dim3(256), 0, (hipStream_t)stream, state, (const T*)u, u_stride,
+                       req_to_state, req_pool_indices, seg_start, seg_len, positions, channels, taps);
+  });
+  MI355_CHECK_LAUNCH("causal_conv_state_update");
+  return MI355_OK;
+}
+
+int mi355_activation(void* out, const void* in, int64_t in_stride, int64_t rows, int64_t cols, int act, int dtype, void* stream) {
+  MI355_REQUIRE(out && in, MI355_ERR_INVALID, "activation: null pointer");
+  MI355_REQUIRE(rows >= 0 && cols > 0 && in_stride >= cols && (act == 1 || act == 2), MI355_ERR_INVALID, "activation: bad shape or kind");
+  if (rows == 0) return MI355_OK;
+  const int grid = (int)std::min<int64_t>((rows * cols + 255) / 256, 256 * 16);
+  MI355_DISPATCH_DTYPE(dtype, "activation", {
+    hipLaunchKernelGGL((activation_kernel<T>), dim3(grid), dim3(256), 0, (hipStream_t)stream, (T*)out, (const T*)in, in_stride, rows,
+                       cols, act);
+  });
+  MI355_CHECK_LAUNCH("activation");
+  return MI355_OK;
+}

@@ -24,7 +24,8 @@ __device__ __forceinline__ float moe_gelu_erf(float z) { return 0.5f * z * (1.0f
 __global__ __launch_bounds__(256) void moe_route_grouped_kernel(int32_t* __restrict__ ids, float* __restrict__ weights,
                                                                 const float* __restrict__ logits,
                                                                 const float* __restrict__ correction, int64_t tokens, int E,
-                                                                int top, int n_groups, int keep, float scale) {
+                                                                int top, int n_groups, int keep, float scale, int score_fn,
+                                                                int group_best, int renorm) {
   extern __shared__ float sm[];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int64_t t = (int64_t)blockIdx.x * 4 + wv;
@@ -34,10 +35,20 @@ __global__ __launch_bounds__(256) void moe_route_grouped_kernel(int32_t* __restr
   const bool valid = t < tokens;
   const int per = E / n_groups;
   if (valid) {
+    float mx = 0.f, inv = 1.f;
+    if (score_fn == 1) {
+      // softmax over all experts
+      mx = -INFINITY;
+      for (int e = lane; e < E; e += 64) mx = fmaxf(mx, logits[t * E + e]);
+      mx = wave_max(mx);
+      float sum = 0.f;
+      for (int e = lane; e < E; e += 64) sum += expf(logits[t * E + e] - mx);
+      inv = 1.0f / wave_sum(sum);
+    }
     for (int e = lane; e < E; e += 64) {
-      const float s = 1.0f / (1.0f + expf(-logits[t * E + e]));
+      const float s = score_fn == 1 ? expf(logits[t * E + e] - mx) * inv : 1.0f / (1.0f + expf(-logits[t * E + e]));
       score[e] = s;
-      choice[e] = s + correction[e];
+      choice[e] = s + (correction != nullptr ? correction[e] : 0.f);
     }
   }
   __syncthreads();
@@ -53,7 +64,7 @@ __global__ __launch_bounds__(256) void moe_route_grouped_kernel(int32_t* __restr
           m2 = c;
         }
       }
-      gsc[g] = per > 1 ? m1 + m2 : m1;
+      gsc[g] = (per > 1 && group_best >= 2) ? m1 + m2 : m1;
     }
   }
   __syncthreads();
@@ -99,7 +110,7 @@ __global__ __launch_bounds__(256) void moe_route_grouped_kernel(int32_t* __restr
     }
   }
   if (lane == 0) {
-    const float inv = scale / (total + 1e-20f);
+    const float inv = renorm ? scale / (total + 1e-20f) : scale;
     for (int k = 0; k < top; ++k) weights[t * top + k] *= inv;
   }
 }
@@ -458,7 +469,17 @@ using namespace mi355;
 
 int mi355_moe_route_grouped(int32_t* ids, float* weights, const float* logits, const float* correction, int64_t tokens,
                             int num_experts, int top, int n_groups, int keep_groups, float scale, void* stream) {
-  MI355_REQUIRE(ids && weights && logits && correction, MI355_ERR_INVALID, "moe_route_grouped: null pointer");
+  MI355_REQUIRE(correction, MI355_ERR_INVALID, "moe_route_grouped: null pointer");
+  return mi355_moe_route_scores(ids, weights, logits, correction, tokens, num_experts, top, n_groups, keep_groups, scale, 0, 2, 1,
+                                stream);
+}
+
+int mi355_moe_route_scores(int32_t* ids, float* weights, const float* logits, const float* correction, int64_t tokens,
+                           int num_experts, int top, int n_groups, int keep_groups, float scale, int score_fn, int group_best,
+                           int renorm, void* stream) {
+  MI355_REQUIRE(ids && weights && logits, MI355_ERR_INVALID, "moe_route_grouped: null pointer");
+  MI355_REQUIRE((score_fn == 0 || score_fn == 1) && (group_best == 1 || group_best == 2), MI355_ERR_INVALID,
+                "moe_route_grouped: scores are sigmoid (0) or softmax (1), a group counts its best 1 or 2");
   MI355_REQUIRE(tokens >= 0 && num_experts > 0 && n_groups > 0 && num_experts % n_groups == 0 && keep_groups >= 1 &&
                     keep_groups <= n_groups && top >= 1 && top <= num_experts / n_groups * keep_groups,
                 MI355_ERR_INVALID, "moe_route_grouped: bad shape");
@@ -466,7 +487,7 @@ int mi355_moe_route_grouped(int32_t* ids, float* weights, const float* logits, c
   if (tokens == 0) return MI355_OK;
   const size_t lds = (size_t)4 * (2 * num_experts + n_groups) * sizeof(float);
   hipLaunchKernelGGL(moe_route_grouped_kernel, dim3((unsigned)((tokens + 3) / 4)), dim3(256), lds, (hipStream_t)stream, ids,
-                     weights, logits, correction, tokens, num_experts, top, n_groups, keep_groups, scale);
+                     weights, logits, correction, tokens, num_experts, top, n_groups, keep_groups, scale, score_fn, group_best, renorm);
   MI355_CHECK_LAUNCH("moe_route_grouped");
   return MI355_OK;
 }

@@ -191,11 +191,12 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(
   }
 }
 
-// One wave per (token, head): out = o / rms(o) (* w) * silu(gate)
+// One wave per (token, head): out = o / rms(o) (* w) * silu(gate), or * sigmoid(gate) with gate_act 1
 template <typename T>
 __global__ __launch_bounds__(256) void head_rmsnorm_gate_kernel(T* __restrict__ out, const float* __restrict__ o,
                                                                 const T* __restrict__ w, const T* __restrict__ gate,
-                                                                int64_t gate_stride, int64_t tokens, int heads, int dv, float eps) {
+                                                                int64_t gate_stride, int64_t tokens, int heads, int dv, float eps,
+                                                                int gate_act) {
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int64_t idx = (int64_t)blockIdx.x * 4 + wv;
   if (idx >= tokens * heads) return;
@@ -211,7 +212,7 @@ __global__ __launch_bounds__(256) void head_rmsnorm_gate_kernel(T* __restrict__ 
   for (int i = lane; i < dv; i += 64) {
     const float z = to_f32(g[i]);
     const float n = r[i] * inv * (w != nullptr ? to_f32(w[i]) : 1.0f);
-    dst[i] = from_f32<T>(n * z * pn_sigmoid(z));
+    dst[i] = from_f32<T>(gate_act == 1 ? n * pn_sigmoid(z) : n * z * pn_sigmoid(z));
   }
 }
 
@@ -224,6 +225,70 @@ __global__ __launch_bounds__(256) void gelu_tanh_mul_rows_kernel(T* __restrict__
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
     const int64_t r = idx / d, i = idx - r * d;
     out[idx] = from_f32<T>(pn_gelu_tanh(to_f32(gate[r * gate_stride + i])) * to_f32(table[ids[r] * table_stride + col_off + i]));
+  }
+}
+
+
+// One workgroup per token: h = x / sqrt(mean(x^2) + eps) * (offset + w)
+template <typename T>
+__global__ __launch_bounds__(256) void offset_rmsnorm_kernel(T* __restrict__ h, const float* __restrict__ x, const T* __restrict__ w,
+                                                             int64_t D, float eps, float offset) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  float q = 0.f;
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    const float v = x[t * D + i];
+    q += v * v;
+  }
+  q = block_sum(q, red);
+  const float inv = 1.0f / sqrtf(q / (float)D + eps);
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) h[t * D + i] = from_f32<T>(x[t * D + i] * inv * (offset + to_f32(w[i])));
+}
+
+// One workgroup per token:  x[t] += s * (A + B) + F,  A = a / rms(a) * wa (wa null: a as it is), B likewise (b null: none),
+// F = f[t], or the sum over j of coef[t][j] * f[rows[t][j]] in that order, or nothing.
+template <typename T>
+__global__ __launch_bounds__(256) void branch_residual_add_kernel(
+    float* __restrict__ x, const T* __restrict__ a, int64_t a_stride, const T* __restrict__ wa, const T* __restrict__ b,
+    int64_t b_stride, const T* __restrict__ wb, float s, const T* __restrict__ f, int64_t f_stride, const int32_t* __restrict__ rows,
+    const float* __restrict__ coef, int n_branch, int64_t D, float eps) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  float inv_a = 1.f, inv_b = 1.f;
+  if (wa != nullptr) {
+    float q = 0.f;
+    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+      const float v = to_f32(a[t * a_stride + i]);
+      q += v * v;
+    }
+    q = block_sum(q, red);
+    inv_a = 1.0f / sqrtf(q / (float)D + eps);
+    __syncthreads();
+  }
+  if (b != nullptr && wb != nullptr) {
+    float q = 0.f;
+    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+      const float v = to_f32(b[t * b_stride + i]);
+      q += v * v;
+    }
+    q = block_sum(q, red);
+    inv_b = 1.0f / sqrtf(q / (float)D + eps);
+  }
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    float m = to_f32(a[t * a_stride + i]) * inv_a * (wa != nullptr ? to_f32(wa[i]) : 1.f);
+    if (b != nullptr) m += to_f32(b[t * b_stride + i]) * inv_b * (wb != nullptr ? to_f32(wb[i]) : 1.f);
+    m *= s;
+    if (f != nullptr) {
+      if (rows == nullptr) {
+        m += to_f32(f[t * f_stride + i]);
+      } else {
+        float e = 0.f;
+        for (int j = 0; j < n_branch; ++j)        // fixed order: the sum does not depend on where the rows lie
+          e += coef[t * n_branch + j] * to_f32(f[(int64_t)rows[t * n_branch + j] * f_stride + i]);
+        m += e;
+      }
+    }
+    x[t * D + i] += m;
   }
 }
 
@@ -296,14 +361,20 @@ int mi355_head_norm_rope(void* out, const void* src, const void* weight, const i
 
 int mi355_head_rmsnorm_gate(void* out, const float* o, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,
                             int heads, int value_dim, float eps, int dtype, void* stream) {
+  return mi355_head_rmsnorm_gate_act(out, o, weight, gate, gate_stride, tokens, heads, value_dim, eps, 0, dtype, stream);
+}
+
+int mi355_head_rmsnorm_gate_act(void* out, const float* o, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,
+                                int heads, int value_dim, float eps, int gate_act, int dtype, void* stream) {
   MI355_REQUIRE(out && o && gate, MI355_ERR_INVALID, "head_rmsnorm_gate: null pointer");
+  MI355_REQUIRE(gate_act == 0 || gate_act == 1, MI355_ERR_INVALID, "head_rmsnorm_gate: the gate is silu (0) or sigmoid (1)");
   MI355_REQUIRE(tokens >= 0 && heads > 0 && value_dim > 0 && gate_stride >= (int64_t)heads * value_dim, MI355_ERR_INVALID,
                 "head_rmsnorm_gate: bad shape");
   if (tokens == 0) return MI355_OK;
   const unsigned grid = (unsigned)((tokens * heads + 3) / 4);
   MI355_DISPATCH_DTYPE(dtype, "head_rmsnorm_gate", {
     hipLaunchKernelGGL((head_rmsnorm_gate_kernel<T>), dim3(grid), dim3(256), 0, (hipStream_t)stream, (T*)out, o, (const T*)weight,
-                       (const T*)gate, gate_stride, tokens, heads, value_dim, eps);
+                       (const T*)gate, gate_stride, tokens, heads, value_dim, eps, gate_act);
   });
   MI355_CHECK_LAUNCH("head_rmsnorm_gate");
   return MI355_OK;
@@ -322,5 +393,37 @@ int mi355_gelu_tanh_mul_rows(void* out, const void* gate, int64_t gate_stride, c
                        gate_stride, (const T*)table, table_stride, col_off, ids, rows, d);
   });
   MI355_CHECK_LAUNCH("gelu_tanh_mul_rows");
+  return MI355_OK;
+}
+
+int mi355_offset_rmsnorm(void* h, const float* x, const void* weight, int64_t tokens, int64_t hidden, float eps, float offset,
+                         int dtype, void* stream) {
+  MI355_REQUIRE(h && x && weight, MI355_ERR_INVALID, "offset_rmsnorm: null pointer");
+  MI355_REQUIRE(tokens >= 0 && hidden > 0, MI355_ERR_INVALID, "offset_rmsnorm: bad shape");
+  if (tokens == 0) return MI355_OK;
+  MI355_DISPATCH_DTYPE(dtype, "offset_rmsnorm", {
+    hipLaunchKernelGGL((offset_rmsnorm_kernel<T>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (T*)h, x,
+                       (const T*)weight, hidden, eps, offset);
+  });
+  MI355_CHECK_LAUNCH("offset_rmsnorm");
+  return MI355_OK;
+}
+
+int mi355_branch_residual_add(float* x, const void* a, int64_t a_stride, const void* wa, const void* b, int64_t b_stride,
+                              const void* wb, float s, const void* f, int64_t f_stride, const int32_t* rows, const float* coef,
+                              int n_branch, int64_t tokens, int64_t hidden, float eps, int dtype, void* stream) {
+  MI355_REQUIRE(x && a, MI355_ERR_INVALID, "branch_residual_add: null pointer");
+  MI355_REQUIRE(tokens >= 0 && hidden > 0 && a_stride >= hidden && (b == nullptr || b_stride >= hidden) &&
+                    (f == nullptr || f_stride >= hidden), MI355_ERR_INVALID, "branch_residual_add: bad shape");
+  MI355_REQUIRE(b != nullptr || wb == nullptr, MI355_ERR_INVALID, "branch_residual_add: a weight without its branch");
+  MI355_REQUIRE((rows == nullptr) == (coef == nullptr) && (rows == nullptr || (f && n_branch > 0)), MI355_ERR_INVALID,
+                "branch_residual_add: rows, coef and their tensor come together");
+  if (tokens == 0) return MI355_OK;
+  MI355_DISPATCH_DTYPE(dtype, "branch_residual_add", {
+    hipLaunchKernelGGL((branch_residual_add_kernel<T>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x, (const T*)a,
+                       a_stride, (const T*)wa, (const T*)b, b_stride, (const T*)wb, s, (const T*)f, f_stride, rows, coef, n_branch,
+                       hidden, eps);
+  });
+  MI355_CHECK_LAUNCH("branch_residual_add");
   return MI355_OK;
 }

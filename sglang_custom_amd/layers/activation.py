@@ -1,4 +1,5 @@
-"""SiluAndMul (python/sglang/srt/layers/activation.py:55-65): x [.., 2d] -> [.., d]."""
+"""SiluAndMul (python/sglang/srt/layers/activation.py:55-65): x [.., 2d] -> [.., d]; Activation: a plain elementwise
+function of a projection's output ("silu", or "relu2", the square of relu)."""
 import torch
 
 from ..custom_op import CustomOp
@@ -18,3 +19,14 @@ class GeluTanhAndMul(CustomOp):
 
     def forward_hip(self, gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
         return get_ops().gelu_tanh_and_mul(gate, up)
+
+
+class Activation(CustomOp):
+    def __init__(self, kind: str):
+        super().__init__()
+        assert kind in ("silu", "relu2")
+        self.kind = kind
+
+    def forward_hip(self, x: torch.Tensor) -> torch.Tensor:
+        """x [T, d] (row-strided: a column block of a wider projection will do) -> contiguous [T, d]."""
+        return get_ops().activation(x, self.kind)

@@ -10,8 +10,15 @@ attention), or one fixed number per head (retention).  The matrices live in the 
 step's tokens of that sequence through it and writes it back, so prefill portions, decode steps and mixed batches are
 the same launch.  Decays, their logarithms and the state are fp32 in every dtype.
 
+GatedDeltaRule: the same hand-off for the delta rule with a decay per key channel,
+
+    S <- diag(a_t) S;   u_t = beta_t (v_t - S^T k_t);   S <- S + k_t u_t^T;   o_t = S^T (q_t * q_scale)
+
+with a_t = exp(-exp(rate_log_h) * softplus(z_t + rate_bias)) from fp32 logits z and beta_t = sigmoid of one logit per head;
+q and k may have fewer heads than v (grouped).
+
 HeadNormGate: the recurrence's fp32 output per head divided by its root mean square (times a weight shared by the heads,
-if there is one), times silu(gate), in the activation dtype for the output projection."""
+if there is one), times silu(gate) or sigmoid(gate), in the activation dtype for the output projection."""
 from typing import Optional
 
 import torch
@@ -41,9 +48,32 @@ class LinearRecurrence(nn.Module):
         return out
 
 
-class HeadNormGate(nn.Module):
-    def __init__(self, value_dim: int, eps: float, dtype, device, with_weight: bool):
+class GatedDeltaRule(nn.Module):
+    def __init__(self, num_heads: int, qk_heads: int, key_dim: int, value_dim: int, layer_id: int, device, q_scale: float = 1.0):
         super().__init__()
+        assert num_heads % qk_heads == 0
+        self.num_heads, self.qk_heads, self.key_dim, self.value_dim, self.layer_id = num_heads, qk_heads, key_dim, value_dim, layer_id
+        self.q_scale = float(q_scale)
+        # fp32 whatever the model dtype: they enter the decay
+        self.rate_log = nn.Parameter(torch.zeros(num_heads, dtype=torch.float32, device=device), requires_grad=False)
+        self.rate_bias = nn.Parameter(torch.zeros(num_heads * key_dim, dtype=torch.float32, device=device), requires_grad=False)
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_logits: torch.Tensor, gate_logits: torch.Tensor,
+                forward_batch):
+        """q, k [T, G, dk], v [T, H, dv], beta_logits [T, H], gate_logits fp32 [T, H * dk] -> fp32 [T, H, dv]."""
+        st = forward_batch.seq_state
+        out = torch.empty((q.shape[0], self.num_heads, self.value_dim), dtype=torch.float32, device=q.device)
+        get_ops().gated_delta_rule(q, k, v, beta_logits, gate_logits, self.rate_bias.data, self.rate_log.data, out,
+                                   st.pool.matrices[self.layer_id], st.req_to_state, st.req_pool_indices, forward_batch.positions,
+                                   self.q_scale, **st.segments())
+        return out
+
+
+class HeadNormGate(nn.Module):
+    def __init__(self, value_dim: int, eps: float, dtype, device, with_weight: bool, gate_act: str = "silu"):
+        super().__init__()
+        assert gate_act in ("silu", "sigmoid")
+        self.gate_act = gate_act
         self.eps = float(eps)
         self.out_dtype = dtype
         self.weight = (nn.Parameter(torch.ones(value_dim, dtype=dtype, device=device), requires_grad=False)
@@ -51,8 +81,10 @@ class HeadNormGate(nn.Module):
 
     def forward(self, o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
         """o fp32 [T, H, dv], gate [T, H * dv] logits (row-strided) -> [T, H * dv]."""
-        return get_ops().head_rmsnorm_gate(o, self.weight.data if self.weight is not None else None, gate, self.eps,
-                                           self.out_dtype)
+        w = self.weight.data if self.weight is not None else None
+        if self.gate_act == "silu":
+            return get_ops().head_rmsnorm_gate(o, w, gate, self.eps, self.out_dtype)
+        return get_ops().head_rmsnorm_gate_act(o, w, gate, self.eps, self.out_dtype, self.gate_act)
 
 
 class HeadNormRope(nn.Module):

@@ -204,12 +204,15 @@ class SequenceStatePool:
     """State that a sequence carries from one step to the next, for models that have such (no counterpart in the
     reference, whose models keep nothing but KV): per slot the last token id, per layer one fp32 row of the
     model's width (the previous token's normed input of a token-shift layer) and, for layers with a linear
-    recurrence, one fp32 matrix per head ([heads, key width, value width], `matrices[layer]`; layers may differ).
+    recurrence, one fp32 matrix per head ([heads, key width, value width], `matrices[layer]`; layers may differ), and
+    for every short causal convolution the last taps - 1 inputs of its channels (`convs[key]`, fp32
+    [slots, taps - 1, channels], row taps - 2 the most recent; the keys are the model's own).
     A request holds one slot from its first prefill portion until it finishes or is retracted; what a freed slot
     holds is never read again, because a sequence's first token (position 0) takes no state.  Slot 0 is never
     handed out."""
 
-    def __init__(self, size: int, layer_num: int, hidden: int, device: str, matrices: Optional[dict] = None):
+    def __init__(self, size: int, layer_num: int, hidden: int, device: str, matrices: Optional[dict] = None,
+                 convs: Optional[dict] = None):
         self.size = size
         self.layer_num = layer_num
         self.hidden = hidden
@@ -218,10 +221,13 @@ class SequenceStatePool:
         self.prev_token = torch.zeros(size + 1, dtype=torch.int32, device=device)
         self.matrices = {layer: torch.zeros((size + 1, h, dk, dv), dtype=torch.float32, device=device)
                          for layer, (h, dk, dv) in (matrices or {}).items()}
+        self.convs = {key: torch.zeros((size + 1, max(taps - 1, 0), channels), dtype=torch.float32, device=device)
+                      for key, (taps, channels) in (convs or {}).items()}
         self.free_slots = list(range(1, size + 1))
 
     def get_state_size_bytes(self) -> int:
-        return self.rows.numel() * 4 + sum(m.numel() * 4 for m in self.matrices.values())
+        return (self.rows.numel() * 4 + sum(m.numel() * 4 for m in self.matrices.values())
+                + sum(c.numel() * 4 for c in self.convs.values()))
 
     def available_size(self) -> int:
         return len(self.free_slots)

@@ -1493,3 +1493,179 @@ def moe_grouped_linear(x: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: 
                                            plan.tile_expert.data_ptr(), plan.n_tiles.data_ptr(), int(gather), int(gelu),
                                            plan.padded, plan.block, N, K, _dt(x), _stream(x)), "moe_grouped_linear")
     return out
+
+
+# ------------------------------------------------------- pre-norm fp32 stream with parallel branches
+def offset_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float = 1.0) -> torch.Tensor:
+    """fp32 rows x [T, D] -> x / sqrt(mean(x^2) + eps) * (offset + weight) in the weight's dtype (a weight stored around zero)."""
+    _gpu(x, weight)
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and weight.is_contiguous() and weight.numel() == x.shape[1]
+    T, D = x.shape
+    h = torch.empty((T, D), dtype=weight.dtype, device=x.device)
+    check(_lib_().mi355_offset_rmsnorm(h.data_ptr(), x.data_ptr(), weight.data_ptr(), T, D, float(eps), float(offset),
+                                       _dt(weight), _stream(x)), "offset_rmsnorm")
+    return h
+
+
+def branch_residual_add(x: torch.Tensor, a: torch.Tensor, wa: Optional[torch.Tensor], b: Optional[torch.Tensor] = None,
+                        wb: Optional[torch.Tensor] = None, s: float = 1.0, f: Optional[torch.Tensor] = None,
+                        rows: Optional[torch.Tensor] = None, coef: Optional[torch.Tensor] = None, eps: float = 1e-6) -> torch.Tensor:
+    """x += s * (A + B) + F in place on the fp32 rows: A = a / rms(a) * wa (wa None: a itself), B likewise from b, wb (b None:
+    nothing), F = f, or sum_j coef[t, j] * f[rows[t, j]] (rows int32 [T, n], coef fp32 [T, n]), or nothing."""
+    _gpu(x, a, wa, b, wb, f, rows, coef)
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous()
+    T, D = x.shape
+    n_branch = 1
+    for y in (a, b):
+        assert y is None or (y.shape == (T, D) and y.stride(1) == 1 and y.dtype == a.dtype)
+    for w in (wa, wb):
+        assert w is None or (w.dtype == a.dtype and w.numel() == D and w.is_contiguous())
+    if f is not None:
+        assert f.dim() == 2 and f.shape[1] == D and f.stride(1) == 1 and f.dtype == a.dtype
+    if rows is not None:
+        assert rows.dtype == torch.int32 and coef.dtype == torch.float32 and rows.shape == coef.shape and rows.shape[0] == T
+        assert rows.is_contiguous() and coef.is_contiguous() and f is not None
+        n_branch = rows.shape[1]
+    else:
+        assert f is None or f.shape[0] == T
+    check(_lib_().mi355_branch_residual_add(x.data_ptr(), a.data_ptr(), a.stride(0), _p(wa), _p(b), b.stride(0) if b is not None else 0,
+                                            _p(wb), float(s), _p(f), f.stride(0) if f is not None else 0, _p(rows), _p(coef),
+                                            n_branch, T, D, float(eps), _dt(a), _stream(x)), "branch_residual_add")
+    return x
+
+
+def head_rmsnorm_gate_act(o: torch.Tensor, weight: Optional[torch.Tensor], gate: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                          gate_act: str = "silu") -> torch.Tensor:
+    """head_rmsnorm_gate with the gate's function chosen: "silu" or "sigmoid"."""
+    _gpu(o, weight, gate)
+    T, H, dv = o.shape
+    assert o.dtype == torch.float32 and o.is_contiguous() and gate.shape == (T, H * dv) and gate.stride(1) == 1
+    assert gate.dtype == out_dtype and (weight is None or (weight.dtype == out_dtype and weight.numel() == dv and weight.is_contiguous()))
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
+    check(_lib_().mi355_head_rmsnorm_gate_act(out.data_ptr(), o.data_ptr(), _p(weight), gate.data_ptr(), gate.stride(0), T, H, dv,
+                                              float(eps), {"silu": 0, "sigmoid": 1}[gate_act], _dt(gate), _stream(o)),
+          "head_rmsnorm_gate")
+    return out
+
+
+ACTIVATIONS = {"none": 0, "silu": 1, "relu2": 2}
+
+
+def causal_conv(u: torch.Tensor, w1: torch.Tensor, state: torch.Tensor, req_to_state: torch.Tensor, req_pool_indices: torch.Tensor,
+                positions: torch.Tensor, w2: Optional[torch.Tensor] = None, residual: bool = False, act: str = "none",
+                tok_req=None, seg_start=None, seg_len=None):
+    """Causal convolution over time per channel of u [T, C] (row-strided) with filter w1 [C, taps] (last column: the current
+    token) and, optionally, a second filter w2 over the same input; with `residual`, u is added to each result; then `act`.
+    Inputs before a step's first token of a sequence come from state[slot] (fp32 [slots, taps - 1, C]; zeros before position
+    0); afterwards the state holds the sequence's last taps - 1 inputs.  Returns y1, or (y1, y2)."""
+    _gpu(u, w1, w2, state, req_to_state, req_pool_indices, positions)
+    T, C = u.shape
+    taps = w1.shape[1]
+    assert u.stride(1) == 1 and w1.shape == (C, taps) and w1.is_contiguous() and w1.dtype == u.dtype
+    assert w2 is None or (w2.shape == w1.shape and w2.is_contiguous() and w2.dtype == u.dtype)
+    assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (taps - 1, C)
+    assert req_to_state.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
+    assert positions.is_contiguous() and positions.numel() == T
+    y1 = torch.empty((T, C), dtype=u.dtype, device=u.device)
+    y2 = torch.empty_like(y1) if w2 is not None else None
+    tr, ss, sl = _seg(tok_req, seg_start, seg_len)
+    assert seg_start is not None or req_pool_indices.numel() == T, "without segments every token is a sequence of its own"
+    lib = _lib_()
+    check(lib.mi355_causal_conv(y1.data_ptr(), _p(y2), u.data_ptr(), u.stride(0), w1.data_ptr(), _p(w2), _p(state) if taps > 1 else None,
+                                req_to_state.data_ptr(), req_pool_indices.data_ptr(), tr, ss, positions.data_ptr(), T, C, taps,
+                                int(bool(residual)), ACTIVATIONS[act], _dt(u), _stream(u)), "causal_conv")
+    if seg_start is not None and taps > 1:
+        check(lib.mi355_causal_conv_state_update(state.data_ptr(), u.data_ptr(), u.stride(0), req_to_state.data_ptr(),
+                                                 req_pool_indices.data_ptr(), ss, sl, positions.data_ptr(), req_pool_indices.numel(),
+                                                 C, taps, _dt(u), _stream(u)), "causal_conv_state_update")
+    return y1 if w2 is None else (y1, y2)
+
+
+def activation(x: torch.Tensor, act: str) -> torch.Tensor:
+    """act(x) over a row-strided [T, d] block, contiguous result: "silu" or "relu2" (the square of relu)."""
+    _gpu(x)
+    T, d = x.shape
+    assert x.stride(1) == 1 and act in ("silu", "relu2")
+    out = torch.empty((T, d), dtype=x.dtype, device=x.device)
+    check(_lib_().mi355_activation(out.data_ptr(), x.data_ptr(), x.stride(0), T, d, ACTIVATIONS[act], _dt(x), _stream(x)), "activation")
+    return out
+
+
+def gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_logits: torch.Tensor, gate_logits: torch.Tensor,
+                     rate_bias: torch.Tensor, rate_log: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
+                     req_to_state: torch.Tensor, req_pool_indices: torch.Tensor, positions: torch.Tensor, q_scale: float,
+                     tok_req=None, seg_start=None, seg_len=None) -> torch.Tensor:
+    """Per head  S = diag(a) S;  u = beta (v - S^T k);  S += k u^T;  out = S^T (q * q_scale)  over every sequence's tokens of the
+    step on state[slot] ([slots, H, dk, dv] fp32).  q, k [T, G, dk] (fp32 or v's dtype; head h reads head h // (H / G)), v
+    [T, H, dv], beta_logits [T, H] (row-strided, v's dtype), gate_logits fp32 [T, H * dk], rate_bias fp32 [H * dk], rate_log
+    fp32 [H]:  a = exp(-exp(rate_log) * softplus(gate_logits + rate_bias)),  beta = sigmoid(beta_logits)."""
+    _gpu(q, k, v, beta_logits, gate_logits, rate_bias, rate_log, out, state, req_to_state, req_pool_indices, positions)
+    T, G, dk = q.shape
+    H, dv = v.shape[1], v.shape[2]
+    assert k.shape == q.shape and v.shape[0] == T and H % G == 0 and q.dtype == k.dtype and q.dtype in (v.dtype, torch.float32)
+    for t in (q, k, v):
+        assert t.stride(2) == 1 and t.stride(1) == t.shape[2], "heads lie side by side in a token's row"
+    assert beta_logits.shape == (T, H) and beta_logits.stride(1) == 1 and beta_logits.dtype == v.dtype
+    assert gate_logits.dtype == torch.float32 and gate_logits.shape == (T, H * dk) and gate_logits.stride(1) == 1
+    assert rate_bias.dtype == torch.float32 and rate_bias.numel() == H * dk and rate_bias.is_contiguous()
+    assert rate_log.dtype == torch.float32 and rate_log.numel() == H and rate_log.is_contiguous()
+    assert out.dtype == torch.float32 and out.shape == (T, H, dv) and out.is_contiguous()
+    assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv)
+    assert req_to_state.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
+    _, ss, sl = _seg(tok_req, seg_start, seg_len)
+    B = req_pool_indices.numel()
+    assert seg_start is not None or B == T, "without segments every token is a sequence of its own"
+    check(_lib_().mi355_gated_delta_rule(out.data_ptr(), state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                         beta_logits.data_ptr(), gate_logits.data_ptr(), rate_bias.data_ptr(), rate_log.data_ptr(),
+                                         req_to_state.data_ptr(), req_pool_indices.data_ptr(), ss, sl, positions.data_ptr(), B, H, G,
+                                         dk, dv, q.stride(0), k.stride(0), v.stride(0), beta_logits.stride(0), gate_logits.stride(0),
+                                         float(q_scale), _dt(q), _dt(v), _stream(q)), "gated_delta_rule")
+    return out
+
+
+def window_attention_block_tokens(heads: int, kv_heads: int, head_dim: int, v_head_dim: int, dtype: torch.dtype) -> int:
+    """Most consecutive tokens of one sequence that a workgroup of window_attention takes."""
+    return int(_lib_().mi355_window_attention_block_tokens(heads, kv_heads, head_dim, v_head_dim, _DT[dtype]))
+
+
+def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, req_to_token: torch.Tensor,
+                     req_pool_indices: torch.Tensor, positions: torch.Tensor, sink: Optional[torch.Tensor], window: int, scale: float,
+                     tok_req=None, blocks=None, max_run: Optional[int] = None) -> torch.Tensor:
+    """Softmax attention of q [T, H, d] over the keys within `window` positions (0: all earlier ones) in caches
+    [slots, G, d] / [slots, G, dv], with exp(sink[h]) added to the denominator (sink fp32 [H] or None) -> out [T, H, dv];
+    blocks int32 [n, 2] runs of at most max_run consecutive tokens of one sequence, or None (one token per run)."""
+    _gpu(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, sink, tok_req, blocks)
+    T, H, d = q.shape
+    G, dv = k_cache.shape[1], v_cache.shape[2]
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape[2] == d and v_cache.shape[1] == G
+    assert out.shape == (T, H, dv) and q.stride(2) == 1 and out.stride(2) == 1 and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
+    assert sink is None or (sink.dtype == torch.float32 and sink.numel() == H and sink.is_contiguous())
+    assert req_to_token.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
+    assert tok_req is None or (tok_req.dtype == torch.int32 and tok_req.numel() == T)
+    if blocks is not None:
+        assert blocks.dtype == torch.int32 and blocks.dim() == 2 and blocks.shape[1] == 2 and blocks.is_contiguous()
+        nb = blocks.shape[0]
+        assert max_run is not None, "runs come with their longest length"
+    else:
+        nb, max_run = T, 1
+    check(_lib_().mi355_window_attention(
+        out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), req_to_token.data_ptr(), req_pool_indices.data_ptr(),
+        _p(tok_req), positions.data_ptr(), _p(blocks), nb, _p(sink), q.stride(0), q.stride(1), out.stride(0), out.stride(1),
+        req_to_token.stride(0), H, G, d, dv, int(window), float(scale), T, int(max_run), _dt(q), _stream(q)), "window_attention")
+    return out
+
+
+def moe_route_scores(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, n_groups: int, keep_groups: int, scale: float,
+                     score_fn: str = "sigmoid", group_best: int = 2, renorm: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
+    """moe_route_grouped with its choices spelled out: scores "sigmoid" or "softmax" (over all experts), an optional
+    selection-only correction, a group scoring the sum of its group_best (1 or 2) best members, weights renormalised or not."""
+    _gpu(logits, correction)
+    T, E = logits.shape
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    assert correction is None or (correction.dtype == torch.float32 and correction.numel() == E)
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    check(_lib_().mi355_moe_route_scores(ids.data_ptr(), w.data_ptr(), logits.data_ptr(), _p(correction), T, E, int(top), int(n_groups),
+                                         int(keep_groups), float(scale), {"sigmoid": 0, "softmax": 1}[score_fn], int(group_best),
+                                         int(bool(renorm)), _stream(logits)), "moe_route_scores")
+    return ids, w

@@ -499,3 +499,146 @@ def gelu_tanh_mul_rows(gate, table, ids, col_off):
     z = gate.float()
     g = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
     return (g * table[ids.long(), col_off: col_off + gate.shape[1]].float()).to(gate.dtype)
+
+
+# ------------------------------------------------------- pre-norm stream with parallel branches, short convolutions, delta rule,
+# windowed attention with a sink.  Token-by-token restatements of what the header says of each kernel; they share nothing
+# with the whole-sequence functions of oracle/gatarax_ref.py that the tests compare against.
+def offset_rmsnorm(x, weight, eps, offset=1.0):
+    return (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * (offset + weight.float())).to(weight.dtype)
+
+
+def branch_residual_add(x, a, wa, b=None, wb=None, s=1.0, f=None, rows=None, coef=None, eps=1e-6):
+    def branch(y, w):
+        y = y.float()
+        return y if w is None else y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps) * w.float()
+    m = branch(a, wa)
+    if b is not None:
+        m = m + branch(b, wb)
+    m = m * s
+    if f is not None:
+        if rows is None:
+            m = m + f.float()
+        else:
+            for t in range(x.shape[0]):
+                for j in range(rows.shape[1]):
+                    m[t] += float(coef[t, j]) * f[int(rows[t, j])].float()
+    x.add_(m)
+    return x
+
+
+def head_rmsnorm_gate_act(o, weight, gate, eps, out_dtype, gate_act="silu"):
+    T, H, dv = o.shape
+    n = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        n = n * weight.float()
+    g = gate.float().reshape(T, H, dv)
+    return (n * (torch.sigmoid(g) if gate_act == "sigmoid" else g * torch.sigmoid(g))).reshape(T, H * dv).to(out_dtype)
+
+
+def _act(z, act):
+    if act == "silu":
+        return z * torch.sigmoid(z)
+    if act == "relu2":
+        return torch.clamp(z, min=0.0) ** 2
+    return z
+
+
+def causal_conv(u, w1, state, req_to_state, req_pool_indices, positions, w2=None, residual=False, act="none", tok_req=None,
+                seg_start=None, seg_len=None):
+    T, C = u.shape
+    taps = w1.shape[1]
+    outs = [torch.empty((T, C), dtype=u.dtype) for _ in range(1 if w2 is None else 2)]
+    hist = None
+    for t, (b, first, last) in enumerate(_segments(T, tok_req, seg_start, seg_len)):
+        slot = int(req_to_state[int(req_pool_indices[b])])
+        if first:
+            # the inputs before this token, oldest first; nothing before position 0
+            hist = [state[slot, i].clone() if int(positions[t]) - (taps - 1 - i) >= 0 else torch.zeros(C) for i in range(taps - 1)]
+        hist.append(u[t].float())
+        for y, w in zip(outs, (w1, w2)):
+            acc = torch.zeros(C)
+            for k in range(taps - 1, -1, -1):
+                acc = acc + w[:, taps - 1 - k].float() * hist[len(hist) - 1 - k]
+            if residual:
+                acc = acc + hist[-1]
+            y[t] = _act(acc, act).to(u.dtype)
+        hist = hist[1:]
+        if last and taps > 1:
+            state[slot] = torch.stack(hist)
+    return outs[0] if w2 is None else tuple(outs)
+
+
+def activation(x, act):
+    return _act(x.float(), act).to(x.dtype).contiguous()
+
+
+def gated_delta_rule(q, k, v, beta_logits, gate_logits, rate_bias, rate_log, out, state, req_to_state, req_pool_indices, positions,
+                     q_scale, tok_req=None, seg_start=None, seg_len=None):
+    T, G, dk = q.shape
+    H = v.shape[1]
+    rep = H // G
+    S = None
+    for t, (b, first, last) in enumerate(_segments(T, tok_req, seg_start, seg_len)):
+        slot = int(req_to_state[int(req_pool_indices[b])])
+        if first:
+            S = torch.zeros_like(state[slot]) if int(positions[t]) == 0 else state[slot].clone()
+        a = torch.exp(-torch.exp(rate_log.float())[:, None] * F.softplus(gate_logits[t].float() + rate_bias.float()).view(H, dk))
+        beta = torch.sigmoid(beta_logits[t].float())
+        kk = k[t].float().repeat_interleave(rep, 0)
+        qq = q[t].float().repeat_interleave(rep, 0) * q_scale
+        S = a[:, :, None] * S
+        u = beta[:, None] * (v[t].float() - torch.einsum("hkv,hk->hv", S, kk))
+        S = S + kk[:, :, None] * u[:, None, :]
+        out[t] = torch.einsum("hkv,hk->hv", S, qq)
+        if last:
+            state[slot] = S
+    return out
+
+
+def window_attention_block_tokens(heads, kv_heads, head_dim, v_head_dim, dtype):
+    return 3
+
+
+def window_attention(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, sink, window, scale, tok_req=None,
+                     blocks=None, max_run=None):
+    T, H, d = q.shape
+    G = k_cache.shape[1]
+    covered = torch.zeros(T, dtype=torch.bool)
+    runs = [(t, 1) for t in range(T)] if blocks is None else [(int(a), int(n)) for a, n in blocks.tolist()]
+    for t0, n in runs:
+        for t in range(t0, t0 + n):
+            assert not covered[t]
+            covered[t] = True
+            b = t if tok_req is None else int(tok_req[t])
+            assert blocks is None or int(tok_req[t0]) == b, "a run crosses two sequences"
+            pos = int(positions[t])
+            lo = max(0, pos - window + 1) if window > 0 else 0
+            slots = req_to_token[int(req_pool_indices[b]), lo: pos + 1].long()
+            kk, vv = k_cache[slots].float(), v_cache[slots].float()
+            for h in range(H):
+                g = h // (H // G)
+                s = (kk[:, g] @ q[t, h].float()) * scale
+                if sink is not None:
+                    s = torch.cat([s, sink[h].float().reshape(1)])
+                p = torch.softmax(s, 0)[: slots.numel()]
+                out[t, h] = (p @ vv[:, g]).to(out.dtype)
+    assert bool(covered.all()), "the runs do not cover every token"
+    return out
+
+
+def moe_route_scores(logits, correction, top, n_groups, keep_groups, scale, score_fn="sigmoid", group_best=2, renorm=True):
+    T, E = logits.shape
+    per = E // n_groups
+    s = torch.softmax(logits.float(), -1) if score_fn == "softmax" else torch.sigmoid(logits.float())
+    c = s + (correction.float() if correction is not None else 0.0)
+    ids = torch.empty((T, top), dtype=torch.int32)
+    w = torch.empty((T, top), dtype=torch.float32)
+    for t in range(T):
+        gs = c[t].view(n_groups, per).topk(min(group_best, per), dim=-1).values.sum(-1)
+        kept = set(sorted(range(n_groups), key=lambda g: (-float(gs[g]), g))[:keep_groups])
+        order = sorted((e for e in range(E) if e // per in kept), key=lambda e: (-float(c[t, e]), e))[:top]
+        ids[t] = torch.tensor(order, dtype=torch.int32)
+        sel = s[t, order]
+        w[t] = (sel / (sel.sum() + 1e-20) if renorm else sel) * scale
+    return ids, w

@@ -1,0 +1,135 @@
+"""Shared pieces of the Gatarax tests: small random models in checkpoint form and the replay of a schedule with every
+logit compared against the whole-sequence oracle (oracle/gatarax_ref.py)."""
+import torch
+
+from oracle import gatarax_ref as ref
+from seturax_util import build_runner, pools_are_whole, random_prompts, rel_err  # noqa: F401  (generic helpers)
+
+
+def parallel(heads=4, kv_heads=2, dim=16, vdim=8, window=5, scale=0.3, conv=3, r_heads=4, r_kv_heads=2, r_dim=8, r_vdim=12,
+             r_conv=4, decay_rank=5, gate_rank=3):
+    return dict(type="parallel",
+                mixer=dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, conv=conv, scale=scale, mask=dict(size=window)),
+                           right=dict(heads=r_heads, kv_heads=r_kv_heads, dim=r_dim, vdim=r_vdim, conv=r_conv)),
+                _ranks=(decay_rank, gate_rank))
+
+
+def lightning(heads=3, dim=8, vdim=12, decay=(0.5, 0.9, 0.99)):
+    return dict(type="lightning", mixer=dict(heads=heads, dim=dim, vdim=vdim, decay=list(decay)))
+
+
+def dense(ff=40):
+    return dict(kind="dense", ff=ff)
+
+
+def moe(experts=6, top=2, count=3, keep=2, ff=20):
+    return dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top, groups=dict(count=count, keep=keep)))
+
+
+def make_config(layers=None, width=48, vocab=53, taps=3, embed_scale=3.0, logit_scale=0.5, eps=1e-5):
+    """layers: list of (mixer spec, mlp spec or None).  The default stacks both mixers and both feed-forwards with unlike sizes."""
+    if layers is None:
+        layers = [(parallel(), dense()), (lightning(), moe()), (parallel(heads=2, kv_heads=1, dim=8, vdim=16, window=9, conv=2,
+                                                                         r_heads=2, r_kv_heads=2, r_dim=12, r_vdim=4, r_conv=3,
+                                                                         decay_rank=2, gate_rank=6), moe(experts=4, top=3, count=1, keep=1)),
+                  (lightning(heads=1, dim=20, vdim=4, decay=(0.8,)), None)]
+    cfg = dict(architecture="Gatarax", vocab=vocab, width=width, logit_scale=logit_scale, norm=dict(eps=eps),
+               embedding=dict(scale=embed_scale), canon=dict(taps=taps),
+               layers=[dict(type=m["type"], mixer={k: (dict(v) if isinstance(v, dict) else v) for k, v in m["mixer"].items()}, mlp=f)
+                       for m, f in layers])
+    cfg["_ranks"] = [m.get("_ranks") for m, _ in layers]      # read by make_weights only
+    return cfg
+
+
+def public(cfg):
+    return {k: v for k, v in cfg.items() if not k.startswith("_")}
+
+
+def make_weights(cfg, seed=0, separated_router=False):
+    """Checkpoint-named tensors with bf16-representable values, so that a bf16 and an fp32 run read the same numbers.
+    separated_router: every router row is a large multiple of one of a few fixed directions mixed into the stream by the
+    embedding, so that the experts' scores lie far apart and no rounding changes which are chosen."""
+    g = torch.Generator().manual_seed(seed)
+    D, V = cfg["width"], cfg["vocab"]
+    taps = cfg["canon"]["taps"]
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (mean + std * torch.randn(*shape, generator=g)).to(torch.bfloat16)
+
+    w = {"embed": rnd(V, D, std=1.0 / cfg["embedding"]["scale"]), "final.norm": rnd(D, std=0.1)}
+    for i, spec in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", spec["mixer"]
+        w[p + "norm1"] = rnd(D, std=0.1)
+        w[p + "canon1"] = rnd(D, taps, std=0.4)
+        if spec["mlp"] is not None:
+            w[p + "canon2"] = rnd(D, taps, std=0.4)
+        if spec["type"] == "parallel":
+            lf, rt = m["left"], m["right"]
+            H, G, d, dv = lf["heads"], lf["kv_heads"], lf["dim"], lf["vdim"]
+            for n, rows in (("q", H * d), ("k", G * d), ("v", G * dv)):
+                w[p + "mix.left." + n] = rnd(rows, D, std=D ** -0.5)
+                w[p + "mix.left." + n + ".b"] = rnd(rows, std=0.3)
+                w[p + "mix.left." + n + ".conv"] = rnd(rows, lf["conv"], std=0.6)
+            w[p + "mix.left.o"] = rnd(D, H * dv, std=(H * dv) ** -0.5)
+            w[p + "mix.left.o.b"] = rnd(D, std=0.3)
+            H, G, d, dv = rt["heads"], rt["kv_heads"], rt["dim"], rt["vdim"]
+            ra, rg = cfg["_ranks"][i]
+            for n, rows in (("q", G * d), ("k", G * d), ("v", H * dv)):
+                w[p + "mix.right." + n] = rnd(rows, D, std=D ** -0.5)
+                w[p + "mix.right." + n + ".conv"] = rnd(rows, rt["conv"], std=0.6)
+            w[p + "mix.right.b"] = rnd(H, D, std=D ** -0.5)
+            w[p + "mix.right.a1"] = rnd(ra, D, std=D ** -0.5)
+            w[p + "mix.right.a2"] = rnd(H * d, ra, std=ra ** -0.5)
+            w[p + "mix.right.dt_bias"] = rnd(H * d, std=0.5, mean=-1.0)
+            w[p + "mix.right.A_log"] = rnd(H, std=0.5)
+            w[p + "mix.right.g1"] = rnd(rg, D, std=D ** -0.5)
+            w[p + "mix.right.g2"] = rnd(H * dv, rg, std=rg ** -0.5)
+            w[p + "mix.right.norm"] = rnd(dv, std=0.1, mean=1.0)
+            w[p + "mix.right.o"] = rnd(D, H * dv, std=(H * dv) ** -0.5)
+            w[p + "mix.left.out"] = rnd(D, std=0.1, mean=1.0)
+            w[p + "mix.right.out"] = rnd(D, std=0.1, mean=1.0)
+        else:
+            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            for n, rows in (("q", H * d), ("k", H * d), ("v", H * dv), ("g", H * dv)):
+                w[p + "mix." + n] = rnd(rows, D, std=D ** -0.5)
+            w[p + "mix.norm"] = rnd(H * dv, std=0.1, mean=1.0)
+            w[p + "mix.o"] = rnd(D, H * dv, std=(H * dv) ** -0.5)
+        mlp = spec["mlp"]
+        if mlp is not None and mlp["kind"] == "dense":
+            w[p + "mlp.up"] = rnd(mlp["ff"], D, std=D ** -0.5)
+            w[p + "mlp.down"] = rnd(D, mlp["ff"], std=mlp["ff"] ** -0.5)
+        elif mlp is not None:
+            E, ff = mlp["router"]["experts"], mlp["expert"]["ff"]
+            w[p + "mlp.router"] = rnd(E, D, std=(4.0 if separated_router else 1.0) * D ** -0.5)
+            for e in range(E):
+                w[f"{p}mlp.e{e}.gate"] = rnd(ff, D, std=D ** -0.5)
+                w[f"{p}mlp.e{e}.up"] = rnd(ff, D, std=D ** -0.5)
+                w[f"{p}mlp.e{e}.down"] = rnd(D, ff, std=ff ** -0.5)
+    return w
+
+
+def replay_and_compare(runner, cfg, weights, prompts, schedule, tol, want_all=None):
+    """schedule: list of steps, each a list of (request name, token count).  Every token's logits are asked for and
+    compared with the oracle's logits of the whole prompt; a request ends with its last token.  Returns the worst error."""
+    from sglang_custom_amd.managers.trace_replay import TraceReplayer
+
+    rp = TraceReplayer(runner)
+    want = want_all if want_all is not None else {k: ref.forward(public(cfg), weights, p) for k, p in prompts.items()}
+    at = {k: 0 for k in prompts}
+    worst = 0.0
+    for step in schedule:
+        entries, rows, end = [], [], []
+        for name, n in step:
+            lo, hi = at[name], at[name] + n
+            entries.append(dict(id=name, tokens=prompts[name][lo:hi], want=list(range(n))))
+            rows.append(want[name][lo:hi])
+            at[name] = hi
+            if hi == len(prompts[name]):
+                end.append(name)
+        got = rp.step(entries, end)
+        e = rel_err(got, torch.cat(rows))
+        assert e < tol, f"step {step}: logits differ from the whole-sequence oracle by {e:.3g} (limit {tol})"
+        worst = max(worst, e)
+    assert all(at[k] == len(p) for k, p in prompts.items()), "the schedule does not cover the prompts"
+    assert not rp.live
+    return worst
