@@ -26,13 +26,22 @@ def moe(experts=6, top=2, count=3, keep=2, ff=20):
     return dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top, groups=dict(count=count, keep=keep)))
 
 
+def default_layers(every_expert=False):
+    """Both mixers and both feed-forwards with unlike sizes.  every_expert: each token uses all experts of its mixtures, so
+    that a 16-bit run and a float64 oracle cannot part ways over a close call between two scores (the weights still
+    differ from token to token)."""
+    a, b = (moe(experts=6, top=6, count=3, keep=3), moe(experts=4, top=4, count=1, keep=1)) if every_expert else \
+           (moe(), moe(experts=4, top=3, count=1, keep=1))
+    return [(parallel(), dense()), (lightning(), a),
+            (parallel(heads=2, kv_heads=1, dim=8, vdim=16, window=9, conv=2, r_heads=2, r_kv_heads=2, r_dim=12, r_vdim=4, r_conv=3,
+                      decay_rank=2, gate_rank=6), b),
+            (lightning(heads=1, dim=20, vdim=4, decay=(0.8,)), None)]
+
+
 def make_config(layers=None, width=48, vocab=53, taps=3, embed_scale=3.0, logit_scale=0.5, eps=1e-5):
-    """layers: list of (mixer spec, mlp spec or None).  The default stacks both mixers and both feed-forwards with unlike sizes."""
+    """layers: list of (mixer spec, mlp spec or None)."""
     if layers is None:
-        layers = [(parallel(), dense()), (lightning(), moe()), (parallel(heads=2, kv_heads=1, dim=8, vdim=16, window=9, conv=2,
-                                                                         r_heads=2, r_kv_heads=2, r_dim=12, r_vdim=4, r_conv=3,
-                                                                         decay_rank=2, gate_rank=6), moe(experts=4, top=3, count=1, keep=1)),
-                  (lightning(heads=1, dim=20, vdim=4, decay=(0.8,)), None)]
+        layers = default_layers()
     cfg = dict(architecture="Gatarax", vocab=vocab, width=width, logit_scale=logit_scale, norm=dict(eps=eps),
                embedding=dict(scale=embed_scale), canon=dict(taps=taps),
                layers=[dict(type=m["type"], mixer={k: (dict(v) if isinstance(v, dict) else v) for k, v in m["mixer"].items()}, mlp=f)
@@ -45,10 +54,8 @@ def public(cfg):
     return {k: v for k, v in cfg.items() if not k.startswith("_")}
 
 
-def make_weights(cfg, seed=0, separated_router=False):
-    """Checkpoint-named tensors with bf16-representable values, so that a bf16 and an fp32 run read the same numbers.
-    separated_router: every router row is a large multiple of one of a few fixed directions mixed into the stream by the
-    embedding, so that the experts' scores lie far apart and no rounding changes which are chosen."""
+def make_weights(cfg, seed=0):
+    """Checkpoint-named tensors with bf16-representable values, so that a bf16 and an fp32 run read the same numbers."""
     g = torch.Generator().manual_seed(seed)
     D, V = cfg["width"], cfg["vocab"]
     taps = cfg["canon"]["taps"]
@@ -100,7 +107,7 @@ def make_weights(cfg, seed=0, separated_router=False):
             w[p + "mlp.down"] = rnd(D, mlp["ff"], std=mlp["ff"] ** -0.5)
         elif mlp is not None:
             E, ff = mlp["router"]["experts"], mlp["expert"]["ff"]
-            w[p + "mlp.router"] = rnd(E, D, std=(4.0 if separated_router else 1.0) * D ** -0.5)
+            w[p + "mlp.router"] = rnd(E, D, std=2.0 * D ** -0.5)
             for e in range(E):
                 w[f"{p}mlp.e{e}.gate"] = rnd(ff, D, std=D ** -0.5)
                 w[f"{p}mlp.e{e}.up"] = rnd(ff, D, std=D ** -0.5)
