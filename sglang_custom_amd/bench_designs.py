@@ -427,3 +427,184 @@ def run_verozen(size: str, dtype: str = "bfloat16", steps: int = 32, prefill_bs:
     out["ff_and_stream_decode"] = verozen_ff_and_stream_kernels(s, decode_bs)
     out["ff_and_stream_prefill"] = verozen_ff_and_stream_kernels(s, prefill_bs * prefill_len)
     return out
+
+
+# ------------------------------------------------------------------------------------------------ Gatarax beside Verozen
+# Gatarax is compared with the package's closest model, Verozen (an fp32 residual stream, attention with grouped key heads
+# over per-layer caches beside recurrent mixers with a matrix per head and sequence, a grouped mixture of experts): same
+# width, depth, vocabulary, attention heads and head widths, recurrent heads, experts and expert width.
+GATARAX_SIZES = {
+    "gx2048": dict(VEROZEN_SIZES["vz2048"], window=1024, taps=4, conv=4, rec_kv_heads=16, low_rank=64),
+    "gx4096": dict(VEROZEN_SIZES["vz4096"], window=1024, taps=4, conv=4, rec_kv_heads=32, low_rank=64),
+    "gxtiny": dict(VEROZEN_SIZES["vztiny"], window=96, taps=4, conv=3, rec_kv_heads=2, low_rank=24),
+}
+
+
+def gatarax_config(s: dict) -> dict:
+    mlp = dict(kind="moe", expert=dict(ff=s["ff"]), router=dict(experts=s["experts"], top=s["top"], groups=dict(count=s["groups"], keep=s["keep"])))
+    par = dict(type="parallel", mlp=mlp,
+               mixer=dict(left=dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], conv=s["conv"], scale=s["dim"] ** -0.5,
+                                    mask=dict(size=s["window"])),
+                          right=dict(heads=s["rec_heads"], kv_heads=s["rec_kv_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"], conv=s["conv"],
+                                     decay_rank=s["low_rank"], gate_rank=s["low_rank"])))
+    lit = dict(type="lightning", mlp=mlp, mixer=dict(heads=s["rec_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"],
+                                                     decay=[0.9 + 0.0123 * (i % 8) for i in range(s["rec_heads"])]))
+    order = [par, lit, par, lit]
+    return dict(architecture="Gatarax", vocab=s["vocab"], width=s["width"], logit_scale=1.0, norm=dict(eps=1e-6), embedding=dict(scale=1.0),
+                canon=dict(taps=s["taps"]), layers=[order[i % 4] for i in range(s["layers"])])
+
+
+def gatarax_mixer_kernels(s: dict, bs: int, ctx: int, prefill_bs: int, prefill_len: int) -> dict:
+    """The token mixers' launches alone, bf16, each beside the closest model's like launch on the same shapes: windowed
+    softmax attention beside sigmoid attention (decode: bytes = every visible key and value row once per sequence; prefill:
+    flops 2 (d + dv) per visible query-key pair and head), the gated delta rule beside the gated linear recurrence (decode:
+    the matrices' bytes, read and written; prefill: fp32 vector flops, 6 per matrix element and token for the plain
+    recurrence, 10 for the delta rule)."""
+    from . import ops
+
+    dev, dt = "cuda", torch.bfloat16
+    H, G, d, W = s["heads"], s["kv_heads"], s["dim"], s["window"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    res = {}
+    slots = bs * ctx + 8
+    kc = torch.randn(slots, G, d, device=dev, generator=g).to(dt)
+    vc = torch.randn(slots, G, d, device=dev, generator=g).to(dt)
+    rtt = (torch.arange(bs * ctx, device=dev, dtype=torch.int32) + 1).view(bs, ctx)
+    rpi = torch.arange(bs, device=dev)
+    q = torch.randn(bs, H, d, device=dev, generator=g).to(dt)
+    o = torch.empty_like(q)
+    sink = torch.zeros(H, device=dev)
+    pos = torch.full((bs,), ctx - 1, device=dev, dtype=torch.int64)
+    t = _timed(lambda: ops.window_attention(q, kc, vc, o, rtt, rpi, pos, sink, W, d ** -0.5), 20)
+    b = bs * min(ctx, W) * G * d * 2 * 2
+    res["gatarax_decode_attention"] = dict(us=round(t * 1e6, 1), gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    temp, bias = torch.ones(H, device=dev), torch.full((H,), -4.0, device=dev)
+    splits = ops.sigmoid_attention_splits(bs, H, G, ctx, dt)
+    t = _timed(lambda: ops.sigmoid_attention(q, kc, vc, o, rtt, rpi, pos, temp, bias, d ** -0.5, num_splits=splits), 20)
+    b = bs * ctx * G * d * 2 * 2
+    res["verozen_decode_attention"] = dict(us=round(t * 1e6, 1), splits=splits, gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    # ---- prefill attention
+    T = prefill_bs * prefill_len
+    kp = torch.randn(T + 8, G, d, device=dev, generator=g).to(dt)
+    vp = torch.randn(T + 8, G, d, device=dev, generator=g).to(dt)
+    rtp = (torch.arange(T, device=dev, dtype=torch.int32) + 1).view(prefill_bs, prefill_len)
+    qp = torch.randn(T, H, d, device=dev, generator=g).to(dt)
+    op = torch.empty_like(qp)
+    posp = torch.arange(prefill_len, device=dev).repeat(prefill_bs)
+    tok_req = torch.repeat_interleave(torch.arange(prefill_bs, device=dev, dtype=torch.int32), prefill_len)
+    rpp = torch.arange(prefill_bs, device=dev)
+    bq = ops.window_attention_block_tokens(H, G, d, d, dt)
+    assert prefill_len % bq == 0
+    starts = torch.arange(0, T, bq, dtype=torch.int32)
+    blocks = torch.stack([starts, torch.full_like(starts, bq)], 1).to(dev)
+    t = _timed(lambda: ops.window_attention(qp, kp, vp, op, rtp, rpp, posp, sink, W, d ** -0.5, tok_req=tok_req, blocks=blocks, max_run=bq), 3)
+    pairs = prefill_bs * sum(min(i + 1, W) for i in range(prefill_len))
+    fl = pairs * H * 2 * 2 * d
+    res["gatarax_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3))
+    bq2 = ops.sigmoid_attention_block_tokens(H, G, d, d, dt)
+    starts = torch.arange(0, T, bq2, dtype=torch.int32)
+    blocks2 = torch.stack([starts, torch.full_like(starts, bq2)], 1).to(dev)
+    t = _timed(lambda: ops.sigmoid_attention(qp, kp, vp, op, rtp, rpp, posp, temp, bias, d ** -0.5, tok_req=tok_req, blocks=blocks2, max_run=bq2), 3)
+    fl = prefill_bs * prefill_len * (prefill_len + 1) // 2 * H * 2 * 2 * d
+    res["verozen_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3))
+    # ---- the recurrences
+    RH, RG, dk, dv = s["rec_heads"], s["rec_kv_heads"], s["rec_dim"], s["rec_vdim"]
+    state = torch.zeros(bs + 1, RH, dk, dv, device=dev)
+    r2s = torch.arange(1, bs + 1, device=dev, dtype=torch.int32)
+    rb, rl = torch.zeros(RH * dk, device=dev), torch.zeros(RH, device=dev)
+    ss = torch.arange(0, T, prefill_len, device=dev, dtype=torch.int32)
+    sl = torch.full((prefill_bs,), prefill_len, device=dev, dtype=torch.int32)
+    for n, seg, reps in ((bs, {}, 20), (T, dict(tok_req=tok_req, seg_start=ss, seg_len=sl), 3)):
+        qd = torch.nn.functional.normalize(torch.randn(n, RG, dk, device=dev, generator=g), dim=-1)
+        kd = torch.nn.functional.normalize(torch.randn(n, RG, dk, device=dev, generator=g), dim=-1)
+        vd = torch.randn(n, RH, dv, device=dev, generator=g).to(dt)
+        be = torch.randn(n, RH, device=dev, generator=g).to(dt)
+        z = torch.randn(n, RH * dk, device=dev, generator=g)
+        od = torch.empty(n, RH, dv, device=dev)
+        rp_, ps_ = (rpi, torch.full((bs,), ctx, device=dev, dtype=torch.int64)) if not seg else (rpp, posp)
+        t = _timed(lambda: ops.gated_delta_rule(qd, kd, vd, be, z, rb, rl, od, state, r2s, rp_, ps_, dk ** -0.5, **seg), reps)
+        qg, kg = (torch.randn(n, RH, dk, device=dev, generator=g).to(dt) for _ in range(2))
+        t2 = _timed(lambda: ops.linear_recurrence(qg, kg, vd, od, state, r2s, rp_, ps_, 1.0, gate_logits=z, tau=8.0, **seg), reps)
+        if not seg:
+            b = bs * RH * dk * dv * 4 * 2
+            res["gatarax_delta_rule_decode"] = dict(us=round(t * 1e6, 1), gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+            res["verozen_gla_decode_recurrence"] = dict(us=round(t2 * 1e6, 1), gbs=round(b / t2 / 1e9), of_hbm_peak=round(b / t2 / HBM_PEAK, 3))
+        else:
+            res["gatarax_delta_rule_prefill"] = dict(ms=round(t * 1e3, 3), vector_tflops=round(T * RH * dk * dv * 10 / t / 1e12, 2),
+                                                     tokens_per_s_per_sequence=round(prefill_len / t))
+            res["verozen_gla_prefill_recurrence"] = dict(ms=round(t2 * 1e3, 3), vector_tflops=round(T * RH * dk * dv * 6 / t2 / 1e12, 2),
+                                                         tokens_per_s_per_sequence=round(prefill_len / t2))
+    return res
+
+
+def gatarax_stream_kernels(s: dict, tokens: int, segments: int) -> dict:
+    """The elementwise launches by bytes moved (bf16 activations, fp32 stream) beside the closest model's norm launch, and
+    the experts' first GEMM with its activation (one launch with erf-GELU there, a GEMM twice as wide plus silu-and-mul here)."""
+    from . import ops
+
+    dev, dt = "cuda", torch.bfloat16
+    D, ff, E, top = s["width"], s["ff"], s["experts"], s["top"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    res = {}
+    x = torch.randn(tokens, D, device=dev, generator=g)
+    w = torch.ones(D, device=dev, dtype=dt)
+    t = _timed(lambda: ops.offset_rmsnorm(x, w, 1e-6, 1.0), 20)
+    res["offset_rmsnorm"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 2) / t / 1e9))
+    h = x.to(dt)
+    taps = s["taps"]
+    w1, w2 = (torch.randn(D, taps, device=dev, generator=g).to(dt) for _ in range(2))
+    state = torch.zeros(segments + 1, taps - 1, D, device=dev)
+    r2s = torch.arange(1, segments + 1, device=dev, dtype=torch.int32)
+    rpi = torch.arange(segments, device=dev)
+    per = tokens // segments
+    if per == 1:
+        seg, pos = {}, torch.full((tokens,), 100, device=dev, dtype=torch.int64)
+    else:
+        seg = dict(tok_req=torch.repeat_interleave(torch.arange(segments, device=dev, dtype=torch.int32), per),
+                   seg_start=torch.arange(0, tokens, per, device=dev, dtype=torch.int32),
+                   seg_len=torch.full((segments,), per, device=dev, dtype=torch.int32))
+        pos = torch.arange(per, device=dev).repeat(segments)
+    t = _timed(lambda: ops.causal_conv(h, w1, state, r2s, rpi, pos, w2=w2, residual=True, **seg), 20)
+    res["causal_conv (two filters, with the state's update)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * 2 * 3 / t / 1e9))
+    a, b, f = (torch.randn(tokens, D, device=dev, generator=g).to(dt) for _ in range(3))
+    t = _timed(lambda: ops.branch_residual_add(x, a, w, b, w, 0.5, f=f), 20)
+    res["branch_residual_add (two normed branches, dense ff)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 4 + 3 * 2) / t / 1e9))
+    big = torch.randn(tokens * top, D, device=dev, generator=g).to(dt)
+    rows = torch.randperm(tokens * top, device=dev, generator=g).to(torch.int32).view(tokens, top)
+    coef = torch.rand(tokens, top, device=dev, generator=g)
+    t = _timed(lambda: ops.branch_residual_add(x, a, w, b, w, 0.5, f=big, rows=rows, coef=coef), 20)
+    res["branch_residual_add (two normed branches, sum of experts)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 4 + (2 + top) * 2) / t / 1e9))
+    t = _timed(lambda: ops.scaled_add_group_rmsnorm(x, f, 3.0, w, s["norm_groups"], 1e-5), 20)
+    res["scaled_add_group_rmsnorm (closest)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 2 + 4 + 2) / t / 1e9))
+    # experts: first GEMM + activation
+    ids, _ = ops.moe_route_scores(torch.randn(tokens, E, device=dev, generator=g), None, top, s["groups"], s["keep"], 1.0, score_fn="softmax",
+                                  group_best=1, renorm=False)
+    t = _timed(lambda: ops.moe_route_scores(torch.zeros(tokens, E, device=dev), None, top, s["groups"], s["keep"], 1.0, score_fn="softmax",
+                                            group_best=1, renorm=False), 10)
+    res["moe_route_scores (softmax; with the fill of its input)"] = dict(us=round(t * 1e6, 1))
+    plan = ops.moe_align(ids, E, wide_ok=True, tiled_ok=tokens > 64)
+    gu_w = (torch.randn(E, 2 * ff, D, device=dev, generator=g) * D ** -0.5).to(dt)
+    up = gu_w[:, :ff].contiguous()
+    t1 = _timed(lambda: ops.silu_and_mul(ops.moe_grouped_linear(h, gu_w, plan, gather=True, gelu=False)), 5)
+    t2 = _timed(lambda: ops.moe_grouped_linear(h, up, plan, gather=True, gelu=True), 5)
+    fl = tokens * top * 2 * ff * D
+    res["moe_block_rows"] = plan.block
+    res["moe_gate_up_silu_mul"] = dict(us=round(t1 * 1e6, 1), tflops=round(2 * fl / t1 / 1e12, 1), of_mfma_peak=round(2 * fl / t1 / MFMA_BF16_PEAK, 3),
+                                       weight_gbs=round(2 * E * ff * D * 2 / t1 / 1e9))
+    res["moe_up_gelu (closest)"] = dict(us=round(t2 * 1e6, 1), tflops=round(fl / t2 / 1e12, 1), of_mfma_peak=round(fl / t2 / MFMA_BF16_PEAK, 3),
+                                        weight_gbs=round(E * ff * D * 2 / t2 / 1e9))
+    return res
+
+
+def run_gatarax(size: str, dtype: str = "bfloat16", steps: int = 32, prefill_bs: int = 4, prefill_len: int = 2048, decode_bs: int = 64,
+                decode_ctx: int = 1024) -> dict:
+    s = GATARAX_SIZES[size]
+    if size == "gxtiny":
+        prefill_bs, prefill_len, decode_bs, decode_ctx = 2, 256, 8, 128
+    out = dict(size=size, shape=s, dtype=dtype, data="synthetic", workload=dict(prefill=[prefill_bs, prefill_len], decode=[decode_bs, decode_ctx], steps=steps))
+    out["gatarax"] = model_throughput(gatarax_config(s), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=False)
+    out["verozen"] = model_throughput(verozen_config(s), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=False)
+    out["mixers"] = gatarax_mixer_kernels(s, decode_bs, decode_ctx, prefill_bs, prefill_len)
+    out["stream_decode"] = gatarax_stream_kernels(s, decode_bs, decode_bs)
+    out["stream_prefill"] = gatarax_stream_kernels(s, prefill_bs * prefill_len, prefill_bs)
+    return out

@@ -115,9 +115,28 @@ def make_weights(cfg, seed=0):
     return w
 
 
+def row_errors(got: torch.Tensor, want: torch.Tensor) -> torch.Tensor:
+    """Per row: rms over the vocabulary of the difference (means taken off) over the rms of the expected row."""
+    d = got.double().cpu() - want.double()
+    d = d - d.mean(-1, keepdim=True)
+    w = want.double() - want.double().mean(-1, keepdim=True)
+    return d.pow(2).mean(-1).sqrt() / w.pow(2).mean(-1).sqrt().clamp_min(1e-9)
+
+
+def within(errors: torch.Tensor, tol: float, sixteen: bool) -> bool:
+    """fp32: every row within tol.  16-bit: every row within 3 tol and all but one in fifty within tol -- a head's output
+    that happens to be near zero (a first token whose query and key are nearly orthogonal, say) is divided by its own root
+    mean square, which turns the rounding of 16-bit projections into a change of direction at that one place."""
+    if not sixteen:
+        return bool(errors.max() < tol)
+    return bool(errors.max() < 3 * tol) and int((errors >= tol).sum()) <= max(1, errors.numel() // 50)
+
+
 def replay_and_compare(runner, cfg, weights, prompts, schedule, tol, want_all=None):
     """schedule: list of steps, each a list of (request name, token count).  Every token's logits are asked for and
     compared with the oracle's logits of the whole prompt; a request ends with its last token.  Returns the worst error."""
+    sixteen = runner.dtype != torch.float32
+    errors = []
     from sglang_custom_amd.managers.trace_replay import TraceReplayer
 
     rp = TraceReplayer(runner)
@@ -134,9 +153,11 @@ def replay_and_compare(runner, cfg, weights, prompts, schedule, tol, want_all=No
             if hi == len(prompts[name]):
                 end.append(name)
         got = rp.step(entries, end)
-        e = rel_err(got, torch.cat(rows))
-        assert e < tol, f"step {step}: logits differ from the whole-sequence oracle by {e:.3g} (limit {tol})"
-        worst = max(worst, e)
+        e = row_errors(got, torch.cat(rows))
+        assert float(e.max()) < (3 * tol if sixteen else tol), f"step {step}: logits differ from the whole-sequence oracle by {float(e.max()):.3g} (limit {tol})"
+        errors.append(e)
+        worst = max(worst, float(e.max()))
     assert all(at[k] == len(p) for k, p in prompts.items()), "the schedule does not cover the prompts"
     assert not rp.live
+    assert within(torch.cat(errors), tol, sixteen), f"{int((torch.cat(errors) >= tol).sum())} of {torch.cat(errors).numel()} rows differ by more than {tol}"
     return worst
