@@ -69,6 +69,114 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(T* __restrict__ y1, T*
   }
 }
 
+// The same for rows of 16-byte channel groups: a thread owns V consecutive channels (V * sizeof(T) = 16) of CONV_TT
+// consecutive tokens, so inputs, filters (V * TAPS consecutive elements) and results move as whole vectors, the filters are
+// read once per CONV_TT tokens, and a token that follows one of its own sequence takes that token's inputs shifted by one
+// instead of reading them again.  TAPS is a template argument so that a filter element's place in its vector is known at
+// compile time.
+constexpr int CONV_TT = 4;
+
+template <typename T, int V, int TAPS>
+__global__ __launch_bounds__(256) void causal_conv_vec_kernel(T* __restrict__ y1, T* __restrict__ y2, const T* __restrict__ u,
+                                                              int64_t u_stride, const T* __restrict__ w1, const T* __restrict__ w2,
+                                                              float* __restrict__ state, const int32_t* __restrict__ req_to_state,
+                                                              const int64_t* __restrict__ req_pool_indices,
+                                                              const int32_t* __restrict__ tok_req, const int32_t* __restrict__ seg_start,
+                                                              const int64_t* __restrict__ positions, int64_t tokens, int64_t C,
+                                                              int residual, int act) {
+  const int64_t groups = C / V;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t tb = idx / groups;
+  if (tb * CONV_TT >= tokens) return;
+  const int64_t c = (idx - tb * groups) * V;
+  float wf[2][V * TAPS];                             // [filter][channel][tap], as stored
+#pragma unroll
+  for (int f = 0; f < 2; ++f) {
+    const T* w = f == 0 ? w1 : w2;
+    if (w == nullptr) break;
+#pragma unroll
+    for (int i = 0; i < TAPS; ++i) {
+      const Vec<T, V> x = ldvec<T, V>(w + c * TAPS + i * V);
+#pragma unroll
+      for (int v = 0; v < V; ++v) wf[f][i * V + v] = to_f32(x.v[v]);
+    }
+  }
+  float in[TAPS][V];                                 // in[k]: the input k tokens back
+#pragma unroll
+  for (int j = 0; j < CONV_TT; ++j) {
+    const int64_t t = tb * CONV_TT + j;
+    if (t >= tokens) break;
+    const int b = tok_req != nullptr ? tok_req[t] : (int)t;
+    const int64_t t0 = seg_start != nullptr ? seg_start[b] : t;
+    const int64_t pos = positions[t];
+    const int back = (int)(t - t0);
+    float* rows = state + (int64_t)req_to_state[req_pool_indices[b]] * (TAPS - 1) * C + c;
+    if (j > 0 && back >= 1) {
+      // the token before is this sequence's and this thread's: its inputs, one further back each
+#pragma unroll
+      for (int k = TAPS - 1; k >= 1; --k)
+#pragma unroll
+        for (int v = 0; v < V; ++v) in[k][v] = in[k - 1][v];
+      const Vec<T, V> x = ldvec<T, V>(u + t * u_stride + c);
+#pragma unroll
+      for (int v = 0; v < V; ++v) in[0][v] = to_f32(x.v[v]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < TAPS; ++k) {
+        if (k <= back) {
+          const Vec<T, V> x = ldvec<T, V>(u + (t - k) * u_stride + c);
+#pragma unroll
+          for (int v = 0; v < V; ++v) in[k][v] = to_f32(x.v[v]);
+        } else if (pos - k >= 0) {
+          const float* r = rows + (int64_t)(TAPS - 1 - (k - back)) * C;
+#pragma unroll
+          for (int v = 0; v < V; v += 4) {
+            const float4 q = *reinterpret_cast<const float4*>(r + v);
+            in[k][v] = q.x; in[k][v + 1] = q.y; in[k][v + 2] = q.z; in[k][v + 3] = q.w;
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < V; ++v) in[k][v] = 0.f;
+        }
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < 2; ++f) {
+      if ((f == 0 ? w1 : w2) == nullptr) break;
+      Vec<T, V> out;
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        float a = 0.f;
+#pragma unroll
+        for (int k = TAPS - 1; k >= 0; --k) a = fmaf(wf[f][v * TAPS + (TAPS - 1 - k)], in[k][v], a);     // oldest tap first
+        if (residual) a += in[0][v];
+        out.v[v] = from_f32<T>(conv_act(a, act));
+      }
+      stvec<T, V>((f == 0 ? y1 : y2) + t * C + c, out);
+    }
+    if (tok_req == nullptr) {
+      // a step of single tokens: this thread is the only reader and writer of its channels' rows
+#pragma unroll
+      for (int k = TAPS - 2; k >= 0; --k) {
+        float* r = rows + (int64_t)(TAPS - 2 - k) * C;
+#pragma unroll
+        for (int v = 0; v < V; v += 4) *reinterpret_cast<float4*>(r + v) = make_float4(in[k][v], in[k][v + 1], in[k][v + 2], in[k][v + 3]);
+      }
+    }
+  }
+}
+
+template <typename T, int TAPS>
+void launch_conv_vec(void* y1, void* y2, const void* u, int64_t u_stride, const void* w1, const void* w2, float* state,
+                     const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* tok_req, const int32_t* seg_start,
+                     const int64_t* positions, int64_t tokens, int64_t channels, int residual, int act, hipStream_t stream) {
+  constexpr int V = 16 / sizeof(T);
+  const int64_t n = ((tokens + CONV_TT - 1) / CONV_TT) * (channels / V);
+  hipLaunchKernelGGL((causal_conv_vec_kernel<T, V, TAPS>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, (T*)y1, (T*)y2,
+                     (const T*)u, u_stride, (const T*)w1, (const T*)w2, state, req_to_state, req_pool_indices, tok_req, seg_start,
+                     positions, tokens, channels, residual, act);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_state_update_kernel(float* __restrict__ state, const T* __restrict__ u,
                                                                        int64_t u_stride, const int32_t* __restrict__ req_to_state,
@@ -121,6 +229,27 @@ int mi355_causal_conv(void* y1, void* y2, const void* u, int64_t u_stride, const
                     act >= 0 && act <= 2, MI355_ERR_INVALID, "causal_conv: bad shape (1 to %d taps)", CONV_MAX_TAPS);
   if (tokens == 0) return MI355_OK;
   MI355_REQUIRE(channels <= 65535 * 256, MI355_ERR_UNSUPPORTED, "causal_conv: too many channels");
+  const int esz = dtype == MI355_F32 ? 4 : 2, vw = 16 / esz;
+  const bool vec = channels % vw == 0 && u_stride % vw == 0 && aligned16(u) && aligned16(y1) && aligned16(w1) &&
+                   (y2 == nullptr || (aligned16(y2) && aligned16(w2))) && (taps == 1 || aligned16(state)) && channels % 4 == 0 &&
+                   tokens * (channels / vw) < ((int64_t)1 << 31) * 256;
+  if (vec) {
+#define MI355_CONV_TAPS(N)                                                                                                    \
+  case N:                                                                                                                     \
+    MI355_DISPATCH_DTYPE(dtype, "causal_conv", {                                                                              \
+      launch_conv_vec<T, N>(y1, y2, u, u_stride, w1, w2, state, req_to_state, req_pool_indices, tok_req, seg_start, positions,   \
+                            tokens, channels, residual, act, (hipStream_t)stream);                                            \
+    });                                                                                                                       \
+    break;
+    switch (taps) {
+      MI355_CONV_TAPS(1) MI355_CONV_TAPS(2) MI355_CONV_TAPS(3) MI355_CONV_TAPS(4) MI355_CONV_TAPS(5) MI355_CONV_TAPS(6)
+      MI355_CONV_TAPS(7) MI355_CONV_TAPS(8)
+      default: break;
+    }
+#undef MI355_CONV_TAPS
+    MI355_CHECK_LAUNCH("causal_conv");
+    return MI355_OK;
+  }
   const dim3 grid((unsigned)tokens, (unsigned)cdiv(channels, 256));
   MI355_DISPATCH_DTYPE(dtype, "causal_conv", {
     hipLaunchKernelGGL((causal_conv_kernel<T>), grid, dim3(256), 0, (hipStream_t)stream, (T*)y1, (T*)y2, (const T*)u, u_stride,

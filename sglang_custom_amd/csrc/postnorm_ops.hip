@@ -246,49 +246,96 @@ __global__ __launch_bounds__(256) void offset_rmsnorm_kernel(T* __restrict__ h, 
 }
 
 // One workgroup per token:  x[t] += s * (A + B) + F,  A = a / rms(a) * wa (wa null: a as it is), B likewise (b null: none),
-// F = f[t], or the sum over j of coef[t][j] * f[rows[t][j]] in that order, or nothing.
-template <typename T>
+// F = f[t], or the sum over j of coef[t][j] * f[rows[t][j]] in that order, or nothing.  VEC: rows move as 16-byte vectors of
+// eight 16-bit (two vectors of four fp32) features; the second pass over a and b finds them in the cache.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void branch_residual_add_kernel(
     float* __restrict__ x, const T* __restrict__ a, int64_t a_stride, const T* __restrict__ wa, const T* __restrict__ b,
     int64_t b_stride, const T* __restrict__ wb, float s, const T* __restrict__ f, int64_t f_stride, const int32_t* __restrict__ rows,
     const float* __restrict__ coef, int n_branch, int64_t D, float eps) {
   __shared__ float red[16];
+  constexpr int W = VEC ? 8 : 1;
   const int64_t t = blockIdx.x;
   float inv_a = 1.f, inv_b = 1.f;
   if (wa != nullptr) {
     float q = 0.f;
-    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-      const float v = to_f32(a[t * a_stride + i]);
-      q += v * v;
+    for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+      if constexpr (VEC) {
+        const Vec<T, 8> v = ld_row8<T>(a + t * a_stride + i);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) q += to_f32(v.v[k]) * to_f32(v.v[k]);
+      } else {
+        const float v = to_f32(a[t * a_stride + i]);
+        q += v * v;
+      }
     }
     q = block_sum(q, red);
     inv_a = 1.0f / sqrtf(q / (float)D + eps);
-    __syncthreads();
   }
   if (b != nullptr && wb != nullptr) {
     float q = 0.f;
-    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-      const float v = to_f32(b[t * b_stride + i]);
-      q += v * v;
+    for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+      if constexpr (VEC) {
+        const Vec<T, 8> v = ld_row8<T>(b + t * b_stride + i);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) q += to_f32(v.v[k]) * to_f32(v.v[k]);
+      } else {
+        const float v = to_f32(b[t * b_stride + i]);
+        q += v * v;
+      }
     }
     q = block_sum(q, red);
     inv_b = 1.0f / sqrtf(q / (float)D + eps);
   }
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-    float m = to_f32(a[t * a_stride + i]) * inv_a * (wa != nullptr ? to_f32(wa[i]) : 1.f);
-    if (b != nullptr) m += to_f32(b[t * b_stride + i]) * inv_b * (wb != nullptr ? to_f32(wb[i]) : 1.f);
-    m *= s;
+  for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+    float m[W];
+    Vec<T, W> va, vb, vwa, vwb, vf;
+    if constexpr (VEC) {
+      va = ld_row8<T>(a + t * a_stride + i);
+      if (wa != nullptr) vwa = ld_row8<T>(wa + i);
+      if (b != nullptr) vb = ld_row8<T>(b + t * b_stride + i);
+      if (wb != nullptr) vwb = ld_row8<T>(wb + i);
+    } else {
+      va.v[0] = a[t * a_stride + i];
+      if (wa != nullptr) vwa.v[0] = wa[i];
+      if (b != nullptr) vb.v[0] = b[t * b_stride + i];
+      if (wb != nullptr) vwb.v[0] = wb[i];
+    }
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      float v = to_f32(va.v[k]) * inv_a * (wa != nullptr ? to_f32(vwa.v[k]) : 1.f);
+      if (b != nullptr) v += to_f32(vb.v[k]) * inv_b * (wb != nullptr ? to_f32(vwb.v[k]) : 1.f);
+      m[k] = v * s;
+    }
     if (f != nullptr) {
       if (rows == nullptr) {
-        m += to_f32(f[t * f_stride + i]);
+        if constexpr (VEC) vf = ld_row8<T>(f + t * f_stride + i); else vf.v[0] = f[t * f_stride + i];
+#pragma unroll
+        for (int k = 0; k < W; ++k) m[k] += to_f32(vf.v[k]);
       } else {
-        float e = 0.f;
-        for (int j = 0; j < n_branch; ++j)        // fixed order: the sum does not depend on where the rows lie
-          e += coef[t * n_branch + j] * to_f32(f[(int64_t)rows[t * n_branch + j] * f_stride + i]);
-        m += e;
+        float e[W];
+#pragma unroll
+        for (int k = 0; k < W; ++k) e[k] = 0.f;
+        for (int j = 0; j < n_branch; ++j) {        // fixed order: the sum does not depend on where the rows lie
+          const float cj = coef[t * n_branch + j];
+          const T* fr = f + (int64_t)rows[t * n_branch + j] * f_stride + i;
+          if constexpr (VEC) vf = ld_row8<T>(fr); else vf.v[0] = fr[0];
+#pragma unroll
+          for (int k = 0; k < W; ++k) e[k] += cj * to_f32(vf.v[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < W; ++k) m[k] += e[k];
       }
     }
-    x[t * D + i] += m;
+    if constexpr (VEC) {
+      float4* xp = reinterpret_cast<float4*>(x + t * D + i);
+      float4 x0 = xp[0], x1 = xp[1];
+      x0.x += m[0]; x0.y += m[1]; x0.z += m[2]; x0.w += m[3];
+      x1.x += m[4]; x1.y += m[5]; x1.z += m[6]; x1.w += m[7];
+      xp[0] = x0; xp[1] = x1;
+    } else {
+      x[t * D + i] += m[0];
+    }
   }
 }
 
@@ -419,10 +466,18 @@ int mi355_branch_residual_add(float* x, const void* a, int64_t a_stride, const v
   MI355_REQUIRE((rows == nullptr) == (coef == nullptr) && (rows == nullptr || (f && n_branch > 0)), MI355_ERR_INVALID,
                 "branch_residual_add: rows, coef and their tensor come together");
   if (tokens == 0) return MI355_OK;
+  const bool vec = hidden % 8 == 0 && aligned16(x) && aligned16(a) && a_stride % 8 == 0 && (wa == nullptr || aligned16(wa)) &&
+                   (b == nullptr || (aligned16(b) && b_stride % 8 == 0)) && (wb == nullptr || aligned16(wb)) &&
+                   (f == nullptr || (aligned16(f) && f_stride % 8 == 0));
   MI355_DISPATCH_DTYPE(dtype, "branch_residual_add", {
-    hipLaunchKernelGGL((branch_residual_add_kernel<T>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x, (const T*)a,
-                       a_stride, (const T*)wa, (const T*)b, b_stride, (const T*)wb, s, (const T*)f, f_stride, rows, coef, n_branch,
-                       hidden, eps);
+    if (vec)
+      hipLaunchKernelGGL((branch_residual_add_kernel<T, true>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x,
+                         (const T*)a, a_stride, (const T*)wa, (const T*)b, b_stride, (const T*)wb, s, (const T*)f, f_stride, rows, coef,
+                         n_branch, hidden, eps);
+    else
+      hipLaunchKernelGGL((branch_residual_add_kernel<T, false>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x,
+                         (const T*)a, a_stride, (const T*)wa, (const T*)b, b_stride, (const T*)wb, s, (const T*)f, f_stride, rows, coef,
+                         n_branch, hidden, eps);
   });
   MI355_CHECK_LAUNCH("branch_residual_add");
   return MI355_OK;

@@ -13,7 +13,7 @@ Per layer (T tokens, width D), besides the GEMMs' own launches:
   ShortCausalConv          (h + C1(h), h + C2(h)): two filters over one input                                1 launch (+ 1 state)
   parallel   in_proj: [left q | k | v | right q | k | v | beta | a1 | g1] in one GEMM (the left part with its biases)
              left    ShortCausalConv on q | k | v; k and v into the cache; WindowSinkAttention; o (with bias)
-             right   ShortCausalConv + silu on q | k | v; unit vectors (q also / sqrt(d)) in fp32; a2(a1) -> fp32 decay
+             right   ShortCausalConv + silu on q | k | v; unit vectors of q | k in fp32 (one launch); a2(a1) -> fp32 decay
                      logits; GatedDeltaRule; g2(g1); HeadNormGate (sigmoid); o
   lightning  in_proj: [q | k | v | g]; silu on q | k | v; LinearRecurrence (fixed decays); HeadNormGate over all heads
              at once (sigmoid); o
@@ -72,11 +72,11 @@ class GataraxParallelMixer(nn.Module):
         self.right_conv = ShortCausalConv(self.right_width, rt["conv"], (layer_id, "right"), dtype, device, act="silu")
         # x / sqrt(sum x^2 + e) = x / sqrt(d) / sqrt(mean x^2 + e / d): the head norm with a unit weight does it
         d = self.rd
-        self.q_unit = HeadNormRope(d, 0, 1.0, True, UNIT_EPS / d, dtype, device, with_norm=True, scale=d ** -0.5 * d ** -0.5)
-        self.k_unit = HeadNormRope(d, 0, 1.0, True, UNIT_EPS / d, dtype, device, with_norm=True, scale=d ** -0.5)
+        # (q and k lie side by side: one launch; q's further factor d^-1/2 rides in the rule's q_scale)
+        self.qk_unit = HeadNormRope(d, 0, 1.0, True, UNIT_EPS / d, dtype, device, with_norm=True, scale=d ** -0.5)
         self.a2 = ReplicatedLinear(decay_rank, self.rH * d, dtype, device)
         self.g2 = ReplicatedLinear(gate_rank, self.rH * self.rdv, dtype, device)
-        self.rule = GatedDeltaRule(self.rH, self.rG, d, self.rdv, layer_id, device)
+        self.rule = GatedDeltaRule(self.rH, self.rG, d, self.rdv, layer_id, device, q_scale=d ** -0.5)
         self.norm_gate = HeadNormGate(self.rdv, eps, dtype, device, with_weight=True, gate_act="sigmoid")
         self.right_o = ReplicatedLinear(self.rH * self.rdv, hidden, dtype, device)
 
@@ -97,8 +97,8 @@ class GataraxParallelMixer(nn.Module):
         # ---- right
         r = self.right_conv(p[:, lw: lw + rw], forward_batch)
         gk = self.rG * self.rd
-        q = self.q_unit(r[:, :gk].view(T, self.rG, self.rd), positions, torch.float32)
-        k = self.k_unit(r[:, gk: 2 * gk].view(T, self.rG, self.rd), positions, torch.float32)
+        qk = self.qk_unit(r[:, : 2 * gk].view(T, 2 * self.rG, self.rd), positions, torch.float32)
+        q, k = qk[:, : self.rG], qk[:, self.rG:]
         v = r[:, 2 * gk:].view(T, self.rH, self.rdv)
         at = lw + rw
         beta = p[:, at: at + self.rH]
@@ -365,7 +365,7 @@ class GataraxForCausalLM(nn.Module):
                 p.data.copy_((0.1 * w).to(p.dtype))
             elif name.endswith("canon.weight") or name.endswith("canon.weight2") or name.endswith("conv.weight"):
                 p.data.copy_((w * p.shape[-1] ** -0.5).to(p.dtype))
-            elif name.endswith("k_unit.weight") or name.endswith("q_unit.weight"):
+            elif name.endswith("qk_unit.weight"):
                 p.data.fill_(1.0)
             elif name.endswith("embed"):
                 p.data.copy_((w / max(self.model.embed_scale, 1e-6)).to(p.dtype))
