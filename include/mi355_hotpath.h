@@ -842,14 +842,16 @@ int mi355_gated_delta_rule(float* out, float* state, const void* q, const void* 
  *   t's sequence with 0 <= pos(t) - j < window (window <= 0: all j <= pos(t)), g = h / (heads / kv_heads); sink null: no
  *   such term.  Caches [slots, kv_heads, head_dim] / [slots, kv_heads, v_head_dim] reached through req_to_token; `blocks`
  *   int32 [num_blocks][2] runs (first token, count <= block_tokens) of consecutive tokens of one sequence, or null (one
- *   token per run); max_run: the longest run.  The new tokens' keys and values must be in the caches already. */
+ *   token per run); max_run: the longest run.  num_splits > 1 (only without `blocks`) cuts every token's keys into that many
+ *   ranges whose partial results (split_scratch: num_splits * tokens * heads * (v_head_dim + 2) floats) a second launch
+ *   merges.  The new tokens' keys and values must be in the caches already. */
 int mi355_window_attention_block_tokens(int heads, int kv_heads, int head_dim, int v_head_dim, int dtype);
 int mi355_window_attention(void* out, const void* q, const void* k_cache, const void* v_cache, const int32_t* req_to_token,
                            const int64_t* req_pool_indices, const int32_t* tok_req, const int64_t* positions,
                            const int32_t* blocks, int64_t num_blocks, const float* sink, int64_t q_token_stride,
                            int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t req_to_token_stride,
-                           int heads, int kv_heads, int head_dim, int v_head_dim, int window, float scale, int64_t tokens,
-                           int max_run, int dtype, void* stream);
+                           int heads, int kv_heads, int head_dim, int v_head_dim, int window, float scale, int num_splits,
+                           float* split_scratch, int64_t tokens, int max_run, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -126,7 +126,7 @@ _SIGNATURES = {
     "mi355_activation": (I, [P, P, L, L, L, I, I, P]),
     "mi355_gated_delta_rule": (I, [P, P, P, P, P, P, P, P, P, P, P, P, P, P, L, I, I, I, I, L, L, L, L, L, F, I, I, P]),
     "mi355_window_attention_block_tokens": (I, [I, I, I, I, I]),
-    "mi355_window_attention": (I, [P, P, P, P, P, P, P, P, P, L, P, L, L, L, L, L, I, I, I, I, I, F, L, I, I, P]),
+    "mi355_window_attention": (I, [P, P, P, P, P, P, P, P, P, L, P, L, L, L, L, L, I, I, I, I, I, F, I, P, L, I, I, P]),
     "mi355_latent_window_attention": (I, [P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, L, L, I, I, I, I, I, F, I, P, L, I, P]),
 }
 

@@ -475,9 +475,10 @@ def gatarax_mixer_kernels(s: dict, bs: int, ctx: int, prefill_bs: int, prefill_l
     o = torch.empty_like(q)
     sink = torch.zeros(H, device=dev)
     pos = torch.full((bs,), ctx - 1, device=dev, dtype=torch.int64)
-    t = _timed(lambda: ops.window_attention(q, kc, vc, o, rtt, rpi, pos, sink, W, d ** -0.5), 20)
+    wsplits = ops.window_attention_splits(bs, H, G, ctx, W, dt)
+    t = _timed(lambda: ops.window_attention(q, kc, vc, o, rtt, rpi, pos, sink, W, d ** -0.5, num_splits=wsplits), 20)
     b = bs * min(ctx, W) * G * d * 2 * 2
-    res["gatarax_decode_attention"] = dict(us=round(t * 1e6, 1), gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    res["gatarax_decode_attention"] = dict(us=round(t * 1e6, 1), splits=wsplits, gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
     temp, bias = torch.ones(H, device=dev), torch.full((H,), -4.0, device=dev)
     splits = ops.sigmoid_attention_splits(bs, H, G, ctx, dt)
     t = _timed(lambda: ops.sigmoid_attention(q, kc, vc, o, rtt, rpi, pos, temp, bias, d ** -0.5, num_splits=splits), 20)

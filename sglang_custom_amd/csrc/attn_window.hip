@@ -11,7 +11,9 @@
 //     LDS rows, the weights through LDS in the activation dtype, P V with V read by columns; a row's rescale factor travels
 //     through LDS from the wave that owns the row's scores to the waves that own its result columns),
 //   * everything else (fp32, odd widths): vector ALU, 16 rows per workgroup, all fp32.
-// Prefill portions, decode steps and mixed batches are the same launch, told apart only by the list of runs.
+// Prefill portions, decode steps and mixed batches are the same launch, told apart only by the list of runs.  A launch of
+// single tokens (a decode step) may cut each token's keys into num_splits ranges: every range leaves its unnormalised sum,
+// running maximum and running sum in fp32 scratch (the sink belongs to the first range), and a second launch merges them.
 #include "common.cuh"
 
 #include <algorithm>
@@ -35,25 +37,28 @@ struct WaArgs {
   const int64_t* positions;
   const int32_t* blocks;
   const float* sink;
+  float* partial;          // num_splits > 1: [split][token][head][dv + 2] = unnormalised result | running max | running sum
   int64_t q_token_stride, q_head_stride, out_token_stride, out_head_stride, req_to_token_stride, tokens;
-  int heads, kv_heads, d, dv, heads_per_tile, window;
+  int heads, kv_heads, d, dv, heads_per_tile, window, num_splits;
   float scale;
 };
 
-// 16 lanes that hold one row: max and sum over them
+// 16 lanes that hold one row (a DPP row): max and sum over them, every lane gets the result.  Lane exchanges inside quads,
+// then across the halves of a half row, then across the row's halves.
+template <int CTRL> __device__ __forceinline__ float wa_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
 __device__ __forceinline__ float row16_max(float x) {
-  x = fmaxf(x, __shfl_xor(x, 1, 64));
-  x = fmaxf(x, __shfl_xor(x, 2, 64));
-  x = fmaxf(x, __shfl_xor(x, 4, 64));
-  x = fmaxf(x, __shfl_xor(x, 8, 64));
-  return x;
+  x = fmaxf(x, wa_dpp<0xB1>(x));      // quad_perm [1,0,3,2]
+  x = fmaxf(x, wa_dpp<0x4E>(x));      // quad_perm [2,3,0,1]
+  x = fmaxf(x, wa_dpp<0x141>(x));     // row_half_mirror
+  return fmaxf(x, wa_dpp<0x140>(x));  // row_mirror
 }
 __device__ __forceinline__ float row16_sum(float x) {
-  x += __shfl_xor(x, 1, 64);
-  x += __shfl_xor(x, 2, 64);
-  x += __shfl_xor(x, 4, 64);
-  x += __shfl_xor(x, 8, 64);
-  return x;
+  x += wa_dpp<0xB1>(x);
+  x += wa_dpp<0x4E>(x);
+  x += wa_dpp<0x141>(x);
+  return x + wa_dpp<0x140>(x);
 }
 
 // Vector-ALU kernel.  sm: Qs [16][d] | Ks [KT][d + 1] | Vs [KT][dv] | Ps [16][KT]
@@ -90,11 +95,14 @@ __global__ __launch_bounds__(256) void window_attention_valu_kernel(WaArgs a) {
   const int first = (int)a.positions[t0];
   const int last = first + nt - 1;                      // the run's tokens are consecutive
   const int lowest = a.window > 0 ? max(0, first - a.window + 1) : 0;
-  const int tile_lo = lowest / WA_KT, tile_hi = last / WA_KT + 1;
+  const int split = blockIdx.z;
+  const int all_lo = lowest / WA_KT, all_hi = last / WA_KT + 1;
+  const int per = (all_hi - all_lo + a.num_splits - 1) / a.num_splits;
+  const int tile_lo = all_lo + split * per, tile_hi = min(all_hi, tile_lo + per);
   const int r = tid >> 4, cx = tid & 15;
   const int hl_r = r % a.heads_per_tile;
   float run_m = WA_NEG, run_l = 0.f;
-  if (a.sink != nullptr) { run_m = a.sink[h0 + min(hl_r, nh - 1)]; run_l = 1.f; }
+  if (a.sink != nullptr && split == 0) { run_m = a.sink[h0 + min(hl_r, nh - 1)]; run_l = 1.f; }
   float acc[16];
 #pragma unroll
   for (int m = 0; m < 16; ++m) acc[m] = 0.f;
@@ -154,6 +162,16 @@ __global__ __launch_bounds__(256) void window_attention_valu_kernel(WaArgs a) {
   }
   const int tl = r / a.heads_per_tile, hl = r - tl * a.heads_per_tile;
   if (tl < nt && hl < nh) {
+    if (a.num_splits > 1) {
+      float* part = a.partial + (((int64_t)split * a.tokens + t0 + tl) * a.heads + h0 + hl) * (dv + 2);
+#pragma unroll
+      for (int m = 0; m < 16; ++m) {
+        const int c = cx + 16 * m;
+        if (c < dv) part[c] = acc[m];
+      }
+      if (cx == 0) { part[dv] = run_m; part[dv + 1] = run_l; }
+      return;
+    }
     const float inv = run_l > 0.f ? 1.0f / run_l : 0.f;
 #pragma unroll
     for (int m = 0; m < 16; ++m) {
@@ -161,6 +179,31 @@ __global__ __launch_bounds__(256) void window_attention_valu_kernel(WaArgs a) {
       if (c >= dv) continue;
       ((T*)a.out)[(t0 + tl) * a.out_token_stride + (int64_t)(h0 + hl) * a.out_head_stride + c] = from_f32<T>(acc[m] * inv);
     }
+  }
+}
+
+// out[t, h] = sum_s acc_s e^(m_s - M) / sum_s l_s e^(m_s - M), M = max_s m_s, over the key ranges in order.  One wave per
+// (token, head).
+template <typename T>
+__global__ __launch_bounds__(256) void window_attention_merge_kernel(T* __restrict__ out, const float* __restrict__ partial,
+                                                                     int64_t tokens, int heads, int dv, int num_splits,
+                                                                     int64_t out_token_stride, int64_t out_head_stride) {
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t idx = (int64_t)blockIdx.x * 4 + wv;
+  if (idx >= tokens * heads) return;
+  const int64_t t = idx / heads;
+  const int h = (int)(idx - t * heads);
+  const int64_t stride = tokens * heads * (int64_t)(dv + 2);
+  const float* p0 = partial + idx * (dv + 2);
+  float M = WA_NEG;
+  for (int k = 0; k < num_splits; ++k) M = fmaxf(M, p0[k * stride + dv]);
+  float L = 0.f;
+  for (int k = 0; k < num_splits; ++k) L += p0[k * stride + dv + 1] * expf(p0[k * stride + dv] - M);
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  for (int c = lane; c < dv; c += 64) {
+    float s = 0.f;
+    for (int k = 0; k < num_splits; ++k) s += p0[k * stride + c] * expf(p0[k * stride + dv] - M);
+    out[t * out_token_stride + (int64_t)h * out_head_stride + c] = from_f32<T>(s * inv);
   }
 }
 
@@ -185,7 +228,7 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
   T* Vs = Ks + WA_KT * qld;
   T* Ps = Vs + WA_KT * vld;
   __shared__ int row_pos[WAM_ROWS];
-  __shared__ float row_alpha[WAM_ROWS], row_l[WAM_ROWS];
+  __shared__ float row_alpha[WAM_ROWS], row_l[WAM_ROWS], row_m[WAM_ROWS];
   const int rep = a.heads / a.kv_heads;
   const int HR = a.heads_per_tile;
   const int chunks = (rep + HR - 1) / HR;
@@ -221,7 +264,10 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
   const int first = (int)a.positions[t0];
   const int last = first + nt - 1;
   const int lowest = a.window > 0 ? max(0, first - a.window + 1) : 0;
-  const int tile_lo = lowest / WA_KT, tile_hi = last / WA_KT + 1;
+  const int split = blockIdx.z;
+  const int all_lo = lowest / WA_KT, all_hi = last / WA_KT + 1;
+  const int per = (all_hi - all_lo + a.num_splits - 1) / a.num_splits;
+  const int tile_lo = all_lo + split * per, tile_hi = min(all_hi, tile_lo + per);
   const int nblk = dv / 16;
   // this lane's four score rows: 16 wv + 4 lg + x
   float run_m[4], run_l[4];
@@ -229,7 +275,7 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
   for (int x = 0; x < 4; ++x) {
     const int r = 16 * wv + 4 * lg + x;
     const int hl = r % HR;
-    if (a.sink != nullptr) { run_m[x] = a.sink[h0 + min(hl, nh - 1)]; run_l[x] = 1.f; }
+    if (a.sink != nullptr && split == 0) { run_m[x] = a.sink[h0 + min(hl, nh - 1)]; run_l[x] = 1.f; }
     else { run_m[x] = WA_NEG; run_l[x] = 0.f; }
   }
   f32x4 acc[4][CT];
@@ -350,7 +396,7 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
   __syncthreads();
   if (li == 0) {
 #pragma unroll
-    for (int x = 0; x < 4; ++x) row_l[16 * wv + 4 * lg + x] = run_l[x];
+    for (int x = 0; x < 4; ++x) { row_l[16 * wv + 4 * lg + x] = run_l[x]; row_m[16 * wv + 4 * lg + x] = run_m[x]; }
   }
   __syncthreads();
 #pragma unroll
@@ -364,6 +410,12 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
         const int r = 16 * rt + 4 * lg + x;
         const int tl = r / HR, hl = r - tl * HR;
         if (tl >= nt || hl >= nh) continue;
+        if (a.num_splits > 1) {
+          float* part = a.partial + (((int64_t)split * a.tokens + t0 + tl) * a.heads + h0 + hl) * (dv + 2);
+          part[col] = acc[rt][c][x];
+          if (col == 0) { part[dv] = row_m[r]; part[dv + 1] = row_l[r]; }
+          continue;
+        }
         const float l = row_l[r];
         ((T*)a.out)[(t0 + tl) * a.out_token_stride + (int64_t)(h0 + hl) * a.out_head_stride + col] =
             from_f32<T>(l > 0.f ? acc[rt][c][x] / l : 0.f);
@@ -423,8 +475,10 @@ int mi355_window_attention(void* out, const void* q, const void* k_cache, const 
                            const int64_t* req_pool_indices, const int32_t* tok_req, const int64_t* positions,
                            const int32_t* blocks, int64_t num_blocks, const float* sink, int64_t q_token_stride,
                            int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t req_to_token_stride,
-                           int heads, int kv_heads, int head_dim, int v_head_dim, int window, float scale, int64_t tokens,
-                           int max_run, int dtype, void* stream) {
+                           int heads, int kv_heads, int head_dim, int v_head_dim, int window, float scale, int num_splits,
+                           float* split_scratch, int64_t tokens, int max_run, int dtype, void* stream) {
+  MI355_REQUIRE(num_splits >= 1 && num_splits <= 64 && (num_splits == 1 || (split_scratch && blocks == nullptr)), MI355_ERR_INVALID,
+                "window_attention: key splits serve launches of one token per run and need scratch");
   MI355_REQUIRE(out && q && k_cache && v_cache && req_to_token && req_pool_indices && positions, MI355_ERR_INVALID,
                 "window_attention: null pointer");
   MI355_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && head_dim > 0 && v_head_dim > 0 && tokens >= 0 &&
@@ -444,17 +498,25 @@ int mi355_window_attention(void* out, const void* q, const void* k_cache, const 
                     aligned16(q) && aligned16(k_cache) && aligned16(v_cache);
   const int rows = mfma ? WAM_ROWS : WA_ROWS;
   a.kv_heads = kv_heads; a.d = head_dim; a.dv = v_head_dim; a.heads_per_tile = wa_heads_per_tile(heads, kv_heads, rows);
-  a.window = window; a.scale = scale;
+  a.window = window; a.scale = scale; a.num_splits = num_splits; a.partial = split_scratch;
   const int tokens_per_tile = std::max(1, rows / a.heads_per_tile);
   MI355_REQUIRE(max_run >= 1 && max_run <= tokens_per_tile, MI355_ERR_UNSUPPORTED,
                 "window_attention: runs of up to %d tokens, this launch takes %d", max_run, tokens_per_tile);
   const int rep = heads / kv_heads;
   const int chunks = (rep + a.heads_per_tile - 1) / a.heads_per_tile;
-  const dim3 grid((unsigned)num_blocks, (unsigned)(kv_heads * chunks));
+  const dim3 grid((unsigned)num_blocks, (unsigned)(kv_heads * chunks), (unsigned)num_splits);
   MI355_REQUIRE(kv_heads * chunks <= 65535, MI355_ERR_UNSUPPORTED, "window_attention: too many heads");
   int rc = MI355_OK;
   MI355_DISPATCH_DTYPE(dtype, "window_attention", { rc = launch_window<T>(a, grid, mfma, (hipStream_t)stream); });
   if (rc != MI355_OK) return rc;
   MI355_CHECK_LAUNCH("window_attention");
+  if (num_splits > 1) {
+    const unsigned g2 = (unsigned)((tokens * heads + 3) / 4);
+    MI355_DISPATCH_DTYPE(dtype, "window_attention", {
+      hipLaunchKernelGGL((window_attention_merge_kernel<T>), dim3(g2), dim3(256), 0, (hipStream_t)stream, (T*)out, split_scratch, tokens,
+                         heads, v_head_dim, num_splits, out_token_stride, out_head_stride);
+    });
+    MI355_CHECK_LAUNCH("window_attention(merge)");
+  }
   return MI355_OK;
 }

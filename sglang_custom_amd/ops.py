@@ -1628,9 +1628,17 @@ def window_attention_block_tokens(heads: int, kv_heads: int, head_dim: int, v_he
     return int(_lib_().mi355_window_attention_block_tokens(heads, kv_heads, head_dim, v_head_dim, _DT[dtype]))
 
 
+def window_attention_splits(tokens: int, heads: int, kv_heads: int, max_len: int, window: int, dtype: torch.dtype) -> int:
+    """Key ranges per token for a decode-sized launch: eight workgroups per CU in flight (a workgroup waits on its own
+    loads; its neighbours' products cover them), at least 128 visible keys each."""
+    wgs = max(1, tokens * kv_heads * ((heads // kv_heads + 63) // 64))
+    seen = min(max_len, window) if window > 0 else max_len
+    return int(max(1, min(64, (2048 + wgs - 1) // wgs, seen // 128)))
+
+
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, req_to_token: torch.Tensor,
                      req_pool_indices: torch.Tensor, positions: torch.Tensor, sink: Optional[torch.Tensor], window: int, scale: float,
-                     tok_req=None, blocks=None, max_run: Optional[int] = None) -> torch.Tensor:
+                     tok_req=None, blocks=None, max_run: Optional[int] = None, num_splits: int = 1) -> torch.Tensor:
     """Softmax attention of q [T, H, d] over the keys within `window` positions (0: all earlier ones) in caches
     [slots, G, d] / [slots, G, dv], with exp(sink[h]) added to the denominator (sink fp32 [H] or None) -> out [T, H, dv];
     blocks int32 [n, 2] runs of at most max_run consecutive tokens of one sequence, or None (one token per run)."""
@@ -1644,14 +1652,16 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     assert tok_req is None or (tok_req.dtype == torch.int32 and tok_req.numel() == T)
     if blocks is not None:
         assert blocks.dtype == torch.int32 and blocks.dim() == 2 and blocks.shape[1] == 2 and blocks.is_contiguous()
-        nb = blocks.shape[0]
+        nb, num_splits = blocks.shape[0], 1
         assert max_run is not None, "runs come with their longest length"
     else:
         nb, max_run = T, 1
+    scratch = torch.empty(num_splits * T * H * (dv + 2), dtype=torch.float32, device=q.device) if num_splits > 1 else None
     check(_lib_().mi355_window_attention(
         out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), req_to_token.data_ptr(), req_pool_indices.data_ptr(),
         _p(tok_req), positions.data_ptr(), _p(blocks), nb, _p(sink), q.stride(0), q.stride(1), out.stride(0), out.stride(1),
-        req_to_token.stride(0), H, G, d, dv, int(window), float(scale), T, int(max_run), _dt(q), _stream(q)), "window_attention")
+        req_to_token.stride(0), H, G, d, dv, int(window), float(scale), int(num_splits), _p(scratch), T, int(max_run), _dt(q), _stream(q)),
+          "window_attention")
     return out
 
 

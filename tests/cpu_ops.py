@@ -600,8 +600,12 @@ def window_attention_block_tokens(heads, kv_heads, head_dim, v_head_dim, dtype):
     return 3
 
 
+def window_attention_splits(tokens, heads, kv_heads, max_len, window, dtype):
+    return 1
+
+
 def window_attention(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, sink, window, scale, tok_req=None,
-                     blocks=None, max_run=None):
+                     blocks=None, max_run=None, num_splits=1):
     T, H, d = q.shape
     G = k_cache.shape[1]
     covered = torch.zeros(T, dtype=torch.bool)

@@ -152,7 +152,7 @@ def check_conv_batch(ops, device, dtype):
 
 
 # ------------------------------------------------------------------------------------------- windowed attention with a sink
-def run_window_attention(ops, device, dtype, q, kn, v, scale, window, cuts, page=1, decode_tail=0, sink=0.0, pad_q=0):
+def run_window_attention(ops, device, dtype, q, kn, v, scale, window, cuts, page=1, decode_tail=0, sink=0.0, pad_q=0, splits=1):
     T, H, d = q.shape
     G = kn.shape[1]
     kv = KVSetup(device, dtype, kn, v, page=page)
@@ -172,20 +172,23 @@ def run_window_attention(ops, device, dtype, q, kn, v, scale, window, cuts, page
         if not decode:
             blocks = torch.tensor([[s, min(bq, n - s)] for s in range(0, n, bq)], dtype=torch.int32, device=device)
         ops.window_attention(qd[at:at + n], kv.k_cache, kv.v_cache, o, kv.tab.req_to_token, b["req_pool_indices"], b["positions"], sk,
-                             window, scale, tok_req=None if decode else b["tok_req"], blocks=blocks, max_run=bq)
+                             window, scale, tok_req=None if decode else b["tok_req"], blocks=blocks, max_run=bq,
+                             num_splits=splits if decode else 1)
         outs.append(o.cpu())
         at += n
     return torch.cat(outs)
 
 
-def check_window_attention(ops, device, dtype, H=4, G=2, d=32, dv=32, T=150, window=40, cuts=(150,), page=1, decode_tail=0, pad_q=0):
+def check_window_attention(ops, device, dtype, H=4, G=2, d=32, dv=32, T=150, window=40, cuts=(150,), page=1, decode_tail=0, pad_q=0,
+                           splits=1):
     g = torch.Generator().manual_seed(3)
     q = _bf(torch.randn(T, H, d, generator=g))
     kn = _bf(torch.randn(T, G, d, generator=g))
     v = _bf(torch.randn(T, G, dv, generator=g))
     scale = 1.7 / math.sqrt(d)
     want = ref.window_sink_attention(q, kn, v, scale, window)
-    got = run_window_attention(ops, device, dtype, q, kn, v, scale, window, cuts, page=page, decode_tail=decode_tail, pad_q=pad_q)
+    got = run_window_attention(ops, device, dtype, q, kn, v, scale, window, cuts, page=page, decode_tail=decode_tail, pad_q=pad_q,
+                               splits=splits)
     _close(got, want, 2e-5 if dtype == torch.float32 else 1.5e-2, f"window attention ({H}/{G} heads of {d}/{dv}) cut into {list(cuts)[:6]}, pages of {page}")
 
 
@@ -193,11 +196,13 @@ def check_window_attention_planted(ops, device, dtype):
     """Scores are zero except where a query and a key are made to meet (score 16): the key exactly window - 1 back is
     seen, the one window back is not, also across a page's border and in decode steps; a far key is out of reach; and a row
     that sees only zero scores gives its n keys the weight 1 / (n + 1) each: the sink counts as one more."""
-    H, G, d, T, window = 2, 1, 32, 300, 72
+    H, G, d, T, W = 2, 1, 32, 300, 56
+    j1, j3 = 120, 128 - (W - 1)            # j1 and j1 + 1 are asked for from j1 + W - 1 and the token after; j3 from 128 and 129
+    a = j1 + W - 1
     q = torch.zeros(T, H, d, dtype=torch.float64)
     kn = torch.zeros(T, G, d, dtype=torch.float64)
     v = torch.zeros(T, G, d, dtype=torch.float64)
-    for j, col in ((2, 0), (120, 1), (121, 2), (57, 3), (299, 4)):
+    for j, col in ((2, 0), (j1, 1), (j1 + 1, 2), (j3, 3), (T - 1, 4)):
         kn[j, 0, col] = 4.0
         v[j, 0, col] = 1.0 + col
 
@@ -205,27 +210,30 @@ def check_window_attention_planted(ops, device, dtype):
         q[i] = 0
         for c in cols:
             q[i, :, c] = 4.0
-    ask(191, [1, 2])       # 191 - 120 = 71 = window - 1: seen; 121 seen too
-    ask(192, [1, 2])       # 192 - 120 = 72: gone; 121 still seen
-    ask(128, [3])          # 128 - 57 = 71: seen, across the border at 64 and 128
+    ask(a, [1, 2])         # a - j1 = window - 1: seen; j1 + 1 seen too
+    ask(a + 1, [1, 2])     # j1 is a whole window back: gone; j1 + 1 still seen
+    ask(128, [3])          # 128 - j3 = window - 1: seen, across the borders at 64 and 128
     ask(129, [3])          # gone
-    ask(299, [0, 4])       # the far key 2 is out of reach, its own key is seen
+    ask(T - 1, [0, 4])     # the far key 2 is out of reach, its own key is seen
     hot = math.exp(16.0)
-    for cuts, tail in (([T], 0), ([190, 1, 1, 1, 107], 0), ([128, 1, 1, 62, 108], 0), ([191, 1, 1, 107], 0), ([298, 1, 1], 2), ([185] + [1] * 10 + [105], 0)):
+    for cuts, tail in (([T], 0), ([a - 1, 1, 1, 1, T - a - 2], 0), ([128, 1, 1, a - 130, T - a], 0), ([a, 1, 1, T - a - 2], 0),
+                       ([T - 2, 1, 1], 2), ([a - 5] + [1] * 10 + [T - a - 5], 0)):
+        assert sum(cuts) == T
         for page in (1, 64):
-            got = run_window_attention(ops, device, dtype, q, kn, v, 1.0, window, cuts, page=page, decode_tail=tail).double()
+            got = run_window_attention(ops, device, dtype, q, kn, v, 1.0, W, cuts, page=page, decode_tail=tail,
+                                       splits=3 if page == 64 else 1).double()
             tol = 1e-5 if dtype == torch.float32 else 1e-2
-            den = 2 * hot + 70 + 1                           # two hot keys, 70 cold ones, the sink
-            assert abs(float(got[191, 0, 1]) - 2.0 * hot / den) < tol and abs(float(got[191, 1, 2]) - 3.0 * hot / den) < tol, (cuts, page)
-            den = hot + 71 + 1
-            assert abs(float(got[192, 0, 1])) < 1e-6 and abs(float(got[192, 0, 2]) - 3.0 * hot / den) < tol, (cuts, page)
+            den = 2 * hot + (W - 2) + 1                      # two hot keys, the cold rest of the window, the sink
+            assert abs(float(got[a, 0, 1]) - 2.0 * hot / den) < tol and abs(float(got[a, 1, 2]) - 3.0 * hot / den) < tol, (cuts, page)
+            den = hot + (W - 1) + 1
+            assert abs(float(got[a + 1, 0, 1])) < 1e-6 and abs(float(got[a + 1, 0, 2]) - 3.0 * hot / den) < tol, (cuts, page)
             assert abs(float(got[128, 1, 3]) - 4.0 * hot / den) < tol and abs(float(got[129, 1, 3])) < 1e-6, (cuts, page)
-            assert abs(float(got[299, 0, 0])) < 1e-6 and abs(float(got[299, 1, 4]) - 5.0 * hot / den) < tol, (cuts, page)
+            assert abs(float(got[T - 1, 0, 0])) < 1e-6 and abs(float(got[T - 1, 1, 4]) - 5.0 * hot / den) < tol, (cuts, page)
             # token 5 sees six keys of score zero, one of which (key 2) holds 1.0 in column 0: 1 / (6 + 1)
             assert abs(float(got[5, 0, 0]) - 1.0 / 7.0) < tol, (cuts, page)
             assert float(got[0].abs().max()) == 0.0 and float(got[1].abs().max()) == 0.0
     # without the sink the same row gives 1 / 6
-    got = run_window_attention(ops, device, dtype, q, kn, v, 1.0, window, [T], sink=None).double()
+    got = run_window_attention(ops, device, dtype, q, kn, v, 1.0, W, [T], sink=None).double()
     assert abs(float(got[5, 0, 0]) - 1.0 / 6.0) < (1e-5 if dtype == torch.float32 else 1e-2)
 
 

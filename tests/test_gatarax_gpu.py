@@ -70,6 +70,9 @@ def test_window_attention_whole_cut_and_decoded(dtype, H, G, d, dv):
         cases.check_window_attention(ops(), DEV, dtype, H=H, G=G, d=d, dv=dv, window=window)
     cases.check_window_attention(ops(), DEV, dtype, H=H, G=G, d=d, dv=dv, window=70, cuts=(60, 3, 2, 85))
     cases.check_window_attention(ops(), DEV, dtype, H=H, G=G, d=d, dv=dv, window=64, cuts=(100,) + (1,) * 50, decode_tail=50, page=16)
+    # decode steps whose keys are cut into ranges that a second launch merges: more ranges than tiles, ranges past the window
+    cases.check_window_attention(ops(), DEV, dtype, H=H, G=G, d=d, dv=dv, window=500, cuts=(100,) + (1,) * 50, decode_tail=50, splits=3)
+    cases.check_window_attention(ops(), DEV, dtype, H=H, G=G, d=d, dv=dv, window=40, cuts=(120,) + (1,) * 30, decode_tail=30, splits=8, page=16)
     cases.check_window_attention(ops(), DEV, dtype, H=H, G=G, d=d, dv=dv, window=20, cuts=(1, 1, 2, 146), pad_q=8)
     cases.check_window_attention(ops(), DEV, dtype, H=H, G=G, d=d, dv=dv, window=9, cuts=(150,), pad_q=3)
 
