@@ -229,20 +229,44 @@ __global__ __launch_bounds__(256) void gelu_tanh_mul_rows_kernel(T* __restrict__
 }
 
 
-// One workgroup per token: h = x / sqrt(mean(x^2) + eps) * (offset + w)
-template <typename T>
+// One workgroup per token: h = x / sqrt(mean(x^2) + eps) * (offset + w).  VEC: eight features per access (two 16-byte loads
+// of the fp32 row, 16-byte weight loads and stores); the second pass over the row finds it in the cache.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void offset_rmsnorm_kernel(T* __restrict__ h, const float* __restrict__ x, const T* __restrict__ w,
                                                              int64_t D, float eps, float offset) {
   __shared__ float red[16];
+  constexpr int W = VEC ? 8 : 1;
   const int64_t t = blockIdx.x;
   float q = 0.f;
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-    const float v = x[t * D + i];
-    q += v * v;
+  for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+    if constexpr (VEC) {
+      const float4 a = *reinterpret_cast<const float4*>(x + t * D + i), b = *reinterpret_cast<const float4*>(x + t * D + i + 4);
+      q += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+    } else {
+      const float v = x[t * D + i];
+      q += v * v;
+    }
   }
   q = block_sum(q, red);
   const float inv = 1.0f / sqrtf(q / (float)D + eps);
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) h[t * D + i] = from_f32<T>(x[t * D + i] * inv * (offset + to_f32(w[i])));
+  for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+    if constexpr (VEC) {
+      const float4 a = *reinterpret_cast<const float4*>(x + t * D + i), b = *reinterpret_cast<const float4*>(x + t * D + i + 4);
+      const float xs[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      const Vec<T, 8> wv = ld_row8<T>(w + i);
+      if constexpr (sizeof(T) == 2) {
+        Vec<T, 8> o;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o.v[k] = from_f32<T>(xs[k] * inv * (offset + to_f32(wv.v[k])));
+        stvec<T, 8>(h + t * D + i, o);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) h[t * D + i + k] = from_f32<T>(xs[k] * inv * (offset + to_f32(wv.v[k])));
+      }
+    } else {
+      h[t * D + i] = from_f32<T>(x[t * D + i] * inv * (offset + to_f32(w[i])));
+    }
+  }
 }
 
 // One workgroup per token:  x[t] += s * (A + B) + F,  A = a / rms(a) * wa (wa null: a as it is), B likewise (b null: none),
@@ -448,9 +472,14 @@ int mi355_offset_rmsnorm(void* h, const float* x, const void* weight, int64_t to
   MI355_REQUIRE(h && x && weight, MI355_ERR_INVALID, "offset_rmsnorm: null pointer");
   MI355_REQUIRE(tokens >= 0 && hidden > 0, MI355_ERR_INVALID, "offset_rmsnorm: bad shape");
   if (tokens == 0) return MI355_OK;
+  const bool vec = hidden % 8 == 0 && aligned16(x) && aligned16(h) && aligned16(weight);
   MI355_DISPATCH_DTYPE(dtype, "offset_rmsnorm", {
-    hipLaunchKernelGGL((offset_rmsnorm_kernel<T>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (T*)h, x,
-                       (const T*)weight, hidden, eps, offset);
+    if (vec)
+      hipLaunchKernelGGL((offset_rmsnorm_kernel<T, true>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (T*)h, x,
+                         (const T*)weight, hidden, eps, offset);
+    else
+      hipLaunchKernelGGL((offset_rmsnorm_kernel<T, false>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (T*)h, x,
+                         (const T*)weight, hidden, eps, offset);
   });
   MI355_CHECK_LAUNCH("offset_rmsnorm");
   return MI355_OK;

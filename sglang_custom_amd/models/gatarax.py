@@ -63,8 +63,6 @@ class GataraxParallelMixer(nn.Module):
         self.in_bias = nn.Parameter(torch.zeros(out, dtype=dtype, device=device), requires_grad=False)
         # left: convolution on [q | k | v], keys and values to the cache, attention, output projection with bias
         self.left_conv = ShortCausalConv(self.left_width, lf["conv"], (layer_id, "left"), dtype, device)
-        self.k_write = HeadNormRope(self.ld, 0, 1.0, True, eps, dtype, device, with_norm=False)
-        self.v_write = HeadNormRope(self.ldv, 0, 1.0, True, eps, dtype, device, with_norm=False)
         self.attn = WindowSinkAttention(self.lH, self.lG, self.ld, self.ldv, lf["scale"], lf["mask"]["size"], layer_id, device)
         self.left_o = ReplicatedLinear(self.lH * self.ldv, hidden, dtype, device)
         self.left_o_bias = nn.Parameter(torch.zeros(hidden, dtype=dtype, device=device), requires_grad=False)
@@ -89,8 +87,7 @@ class GataraxParallelMixer(nn.Module):
         c = self.left_conv(p[:, :lw], forward_batch)
         nq, nk = self.lH * self.ld, self.lG * self.ld
         k_cache, v_cache = forward_batch.token_to_kv_pool.get_kv_buffer(self.attn.layer_id)
-        self.k_write(c[:, nq: nq + nk].view(T, self.lG, self.ld), positions, h.dtype, cache=k_cache, loc=forward_batch.out_cache_loc)
-        self.v_write(c[:, nq + nk:].view(T, self.lG, self.ldv), positions, h.dtype, cache=v_cache, loc=forward_batch.out_cache_loc)
+        ops.set_kv_buffer(k_cache, v_cache, forward_batch.out_cache_loc, c[:, nq: nq + nk], c[:, nq + nk:])      # both in one launch
         o = torch.empty((T, self.lH, self.ldv), dtype=h.dtype, device=h.device)
         self.attn(c[:, :nq].view(T, self.lH, self.ld), forward_batch, o)
         left = self.left_o.quant_method.apply(self.left_o, o.view(T, self.lH * self.ldv), self.left_o_bias.data)
