@@ -235,6 +235,14 @@ def check_window_attention_planted(ops, device, dtype):
     # without the sink the same row gives 1 / 6
     got = run_window_attention(ops, device, dtype, q, kn, v, 1.0, W, [T], sink=None).double()
     assert abs(float(got[5, 0, 0]) - 1.0 / 6.0) < (1e-5 if dtype == torch.float32 else 1e-2)
+    # a window wider than the sequence (and no window at all): the far key 2 is one hot key among hundreds for the last token,
+    # whole, cut, and decoded over key ranges
+    for window in (T + 50, 0):
+        for cuts, tail, splits in (([T], 0, 1), ([3, 2, T - 6, 1], 0, 1), ([T - 1, 1], 1, 4)):
+            got = run_window_attention(ops, device, dtype, q, kn, v, 1.0, window, cuts, page=64, decode_tail=tail, splits=splits).double()
+            den = 2 * hot + (T - 2) + 1
+            tol = 1e-5 if dtype == torch.float32 else 1e-2
+            assert abs(float(got[T - 1, 0, 0]) - 1.0 * hot / den) < tol and abs(float(got[T - 1, 1, 4]) - 5.0 * hot / den) < tol, (window, cuts)
 
 
 # ------------------------------------------------------------------------------------------- gated delta rule

@@ -186,6 +186,35 @@ def test_long_decode_on_other_sizes(dtype, tol, page_size):
 
 
 @pytest.mark.parametrize("dtype,tol", CASES)
+def test_sizes_that_are_multiples_of_nothing_in_particular(dtype, tol):
+    """Five layers in another order, without feed-forward at the end: attention heads of 48 with values of 80 (the
+    vector-ALU kernel in bf16 too) and of 128 / 128, 8 query heads on 2 key heads, windows of 7, 33 and 200, convolutions
+    of 2 to 5 taps, delta-rule heads of 24 x 40 on shared keys and of 128 x 128, five decays incl. 1, eight experts in four
+    groups, a width of 192; a 260-token prompt beside shorter ones, portions beside single tokens, the pools used twice."""
+    every = dtype != "float32"
+    layers = [(gu.lightning(heads=5, dim=48, vdim=24, decay=(0.5, 0.9, 0.99, 0.999, 1.0)),
+               gu.moe(experts=8, top=8 if every else 3, count=4, keep=4 if every else 2, ff=40)),
+              (gu.parallel(heads=8, kv_heads=2, dim=48, vdim=80, window=33, scale=0.2, conv=2, r_heads=6, r_kv_heads=3, r_dim=24, r_vdim=40,
+                           r_conv=5, decay_rank=12, gate_rank=20), gu.dense(100)),
+              (gu.parallel(heads=4, kv_heads=4, dim=128, vdim=128, window=200, scale=0.09, conv=4, r_heads=2, r_kv_heads=1, r_dim=128,
+                           r_vdim=128, r_conv=4, decay_rank=24, gate_rank=24), gu.moe(experts=4, top=4 if every else 2, count=2, keep=2, ff=96)),
+              (gu.lightning(heads=8, dim=32, vdim=32, decay=[0.9 + 0.01 * i for i in range(8)]), None),
+              (gu.parallel(heads=3, kv_heads=1, dim=64, vdim=32, window=7, scale=0.125, conv=3, r_heads=3, r_kv_heads=3, r_dim=64, r_vdim=64,
+                           r_conv=3, decay_rank=8, gate_rank=8), None)]
+    cfg = gu.make_config(layers=layers, width=192, vocab=1000, taps=2, embed_scale=9.0, logit_scale=0.1, eps=1e-6)
+    w = gu.make_weights(cfg, seed=5)
+    mr = gu.build_runner(cfg, w, dtype=dtype, device=DEV, max_total_tokens=448, max_running_requests=4)
+    p = gu.random_prompts(cfg, [260, 90, 3, 60], seed=8)
+    want = {k: ref.forward(gu.public(cfg), w, x) for k, x in p.items()}
+    gu.replay_and_compare(mr, cfg, w, {"r0": p["r0"]}, [[("r0", 260)]], tol, want_all=want)
+    sched = [[("r0", 64), ("r1", 64), ("r2", 2)], [("r0", 29), ("r1", 2), ("r2", 1), ("r3", 16)], [("r0", 128), ("r1", 3), ("r3", 3)],
+             [("r0", 2), ("r1", 16), ("r3", 35)], [("r0", 30), ("r1", 4), ("r3", 5)]] + [[("r0", 1), ("r1", 1), ("r3", 1)]] + [[("r0", 1)]] * 6
+    for _ in range(2):
+        gu.replay_and_compare(mr, cfg, w, p, sched, tol, want_all=want)
+        assert gu.pools_are_whole(mr)
+
+
+@pytest.mark.parametrize("dtype,tol", CASES)
 def test_equal_and_unit_sizes(dtype, tol):
     """The sizes of the CPU test of this name, with heads of 8 where it has heads of 4: a head of 4 values divided by its
     root mean square turns bf16 noise into a large change of direction whenever the head's output is near zero."""
