@@ -853,6 +853,80 @@ int mi355_window_attention(void* out, const void* q, const void* k_cache, const 
                            int heads, int kv_heads, int head_dim, int v_head_dim, int window, float scale, int num_splits,
                            float* split_scratch, int64_t tokens, int max_run, int dtype, void* stream);
 
+/* ---- the same kernels with further constants as arguments --------------------------------------------
+ * mi355_rmsnorm_residual_add_scaled: x[t] += mult * layer_scale * y[t] / sqrt(mean(y[t]^2) + eps) * (offset + weight); layer_scale
+ *   [hidden] of y's type (null: ones); h_out (T, may be null) = the new x.
+ * mi355_head_norm_rope_mag: mi355_head_norm_rope with cos and sin multiplied by rot_mag (frequencies scaled for longer
+ *   sequences come with such a magnitude; the frequencies themselves are the caller's table).
+ * mi355_gated_group_rmsnorm: out[t] = N(y[t] * silu(gate[t])) * weight, N over `groups` equal consecutive parts of the row,
+ *   the gate applied before the norm; y fp32 [tokens, hidden] contiguous, gate T row-strided, out T contiguous.
+ * mi355_causal_conv_bias: mi355_causal_conv with bias1 [channels] (null: none) added to the first filter's sum before act.
+ * mi355_linear_recurrence_ssm: mi355_linear_recurrence with q, k [tokens, qk_heads, key_dim] (head h reads head
+ *   h / (heads / qk_heads)) and a third kind of decay: dt = softplus(dt_logits[t * dt_token_stride + h] + dt_bias[h]),
+ *   a = exp(-exp(rate_log[h]) * dt) for every key channel, S = a S + dt k v^T, out = S^T (q * q_scale) + skip[h] v (skip null:
+ *   none).  Exactly one of gate_logits, head_decay, dt_logits is given.
+ * mi355_gated_delta_rule_ex: mi355_gated_delta_rule with gate_per_head (gate_logits [tokens][heads], rate_bias [heads]: one
+ *   decay per head and token) and beta_f32 (beta_logits are fp32). */
+int mi355_rmsnorm_residual_add_scaled(float* x, void* h_out, const void* y, int64_t y_stride, const void* weight,
+                                      const void* layer_scale, float offset, float mult, int64_t tokens, int64_t hidden, float eps,
+                                      int dtype, void* stream);
+int mi355_head_norm_rope_mag(void* out, const void* src, const void* weight, const int64_t* positions, const int64_t* loc,
+                             const float* inv_freq, int64_t tokens, int heads, int head_dim, int64_t src_token_stride,
+                             int64_t src_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t out_rows,
+                             int rot_dims, int interleaved, float scale, float eps, float rot_mag, int dtype, int out_dtype,
+                             void* stream);
+/* mi355_qkv_norm_rope_write: the three head norms of an attention layer in one launch: q [tokens][heads][head_dim], k
+ *   [tokens][kv_heads][head_dim], v [tokens][kv_heads][v_head_dim] (heads side by side in a token's row, token strides given).
+ *   q: RMS norm with wq, rotation as mi355_head_norm_rope_mag, to q_out [tokens][heads][head_dim] contiguous; k: the same with
+ *   wk, into k_cache[loc[t]] ([slots][kv_heads][head_dim]); v: divided by sqrt(mean(v^2) + eps), into v_cache[loc[t]]. */
+int mi355_qkv_norm_rope_write(void* q_out, void* k_cache, void* v_cache, const void* q, const void* k, const void* v,
+                              int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, const void* wq, const void* wk,
+                              const int64_t* positions, const int64_t* loc, const float* inv_freq, int64_t tokens, int heads,
+                              int kv_heads, int head_dim, int v_head_dim, int rot_dims, int interleaved, float eps, float rot_mag,
+                              int dtype, void* stream);
+int mi355_gated_group_rmsnorm(void* out, const float* y, const void* gate, int64_t gate_stride, const void* weight, int64_t tokens,
+                              int64_t hidden, int groups, float eps, int dtype, void* stream);
+int mi355_causal_conv_bias(void* y1, void* y2, const void* u, int64_t u_stride, const void* w1, const void* w2, const void* bias1,
+                           float* state, const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* tok_req,
+                           const int32_t* seg_start, const int64_t* positions, int64_t tokens, int64_t channels, int taps,
+                           int residual, int act, int dtype, void* stream);
+int mi355_linear_recurrence_ssm(float* out, float* state, const void* q, const void* k, const void* v, const float* gate_logits,
+                                const void* gate_bias, const float* head_decay, const float* dt_logits, int64_t dt_token_stride,
+                                const float* dt_bias, const float* rate_log, const float* skip, const int32_t* req_to_state,
+                                const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                                const int64_t* positions, int64_t batch, int heads, int qk_heads, int key_dim, int value_dim,
+                                int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, int64_t gate_token_stride,
+                                float q_scale, float tau, int qk_dtype, int v_dtype, void* stream);
+int mi355_gated_delta_rule_ex(float* out, float* state, const void* q, const void* k, const void* v, const void* beta_logits,
+                              const float* gate_logits, const float* rate_bias, const float* rate_log, const int32_t* req_to_state,
+                              const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                              const int64_t* positions, int64_t batch, int heads, int qk_heads, int key_dim, int value_dim,
+                              int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, int64_t beta_token_stride,
+                              int64_t gate_token_stride, float q_scale, int gate_per_head, int beta_f32, int qk_dtype, int v_dtype,
+                              void* stream);
+
+/* ---- window attention with averaged blocks before the window and a gate per head -------------------------
+ * mi355_pool_kv_blocks: for every token t of the step whose position p ends a block of `pool` tokens ((p + 1) % pool == 0):
+ *   pooled_k[slot(p) / pool_div][g] = mean over j = p - pool + 1 .. p of k_cache[slot(j)][g] (summed in that order in fp32),
+ *   the same for the values; slot(j) = req_to_token[row of t's sequence][j].  The step's keys and values must be in the
+ *   caches already.  pool_div: 1, or `pool` when pages are whole multiples of `pool` slots (then a block's slots are
+ *   consecutive and the pooled buffers hold one row per `pool` slots).
+ * mi355_window_attention_pooled: mi355_window_attention where token t also sees, for every block b with
+ *   b * pool + pool - 1 <= pos(t) - window, the pooled key / value row of that block (same softmax), and where head h's
+ *   result is multiplied by sigmoid(head_gate[t * gate_token_stride + h]) (T; null: no gate).  pool 0: no blocks. */
+int mi355_pool_kv_blocks(void* pooled_k, void* pooled_v, const void* k_cache, const void* v_cache, const int32_t* req_to_token,
+                         const int64_t* req_pool_indices, const int32_t* tok_req, const int64_t* positions, int64_t tokens,
+                         int64_t req_to_token_stride, int kv_heads, int head_dim, int v_head_dim, int pool, int pool_div, int dtype,
+                         void* stream);
+int mi355_window_attention_pooled(void* out, const void* q, const void* k_cache, const void* v_cache, const void* pooled_k,
+                                  const void* pooled_v, const int32_t* req_to_token, const int64_t* req_pool_indices,
+                                  const int32_t* tok_req, const int64_t* positions, const int32_t* blocks, int64_t num_blocks,
+                                  const float* sink, const void* head_gate, int64_t gate_token_stride, int64_t q_token_stride,
+                                  int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride,
+                                  int64_t req_to_token_stride, int heads, int kv_heads, int head_dim, int v_head_dim, int window,
+                                  int pool, int pool_div, float scale, int num_splits, float* split_scratch, int64_t tokens,
+                                  int max_run, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -127,6 +127,15 @@ _SIGNATURES = {
     "mi355_gated_delta_rule": (I, [P, P, P, P, P, P, P, P, P, P, P, P, P, P, L, I, I, I, I, L, L, L, L, L, F, I, I, P]),
     "mi355_window_attention_block_tokens": (I, [I, I, I, I, I]),
     "mi355_window_attention": (I, [P, P, P, P, P, P, P, P, P, L, P, L, L, L, L, L, I, I, I, I, I, F, I, P, L, I, I, P]),
+    "mi355_rmsnorm_residual_add_scaled": (I, [P, P, P, L, P, P, F, F, L, L, F, I, P]),
+    "mi355_head_norm_rope_mag": (I, [P, P, P, P, P, P, L, I, I, L, L, L, L, L, I, I, F, F, F, I, I, P]),
+    "mi355_qkv_norm_rope_write": (I, [P, P, P, P, P, P, L, L, L, P, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P]),
+    "mi355_gated_group_rmsnorm": (I, [P, P, P, L, P, L, L, I, F, I, P]),
+    "mi355_causal_conv_bias": (I, [P, P, P, L, P, P, P, P, P, P, P, P, P, L, L, I, I, I, I, P]),
+    "mi355_linear_recurrence_ssm": (I, [P, P, P, P, P, P, P, P, P, L, P, P, P, P, P, P, P, P, L, I, I, I, I, L, L, L, L, F, F, I, I, P]),
+    "mi355_gated_delta_rule_ex": (I, [P, P, P, P, P, P, P, P, P, P, P, P, P, P, L, I, I, I, I, L, L, L, L, L, F, I, I, I, I, P]),
+    "mi355_pool_kv_blocks": (I, [P, P, P, P, P, P, P, P, L, L, I, I, I, I, I, I, P]),
+    "mi355_window_attention_pooled": (I, [P, P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, I, I, I, I, I, I, I, F, I, P, L, I, I, P]),
     "mi355_latent_window_attention": (I, [P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, L, L, I, I, I, I, I, F, I, P, L, I, P]),
 }
 

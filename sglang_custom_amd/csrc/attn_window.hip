@@ -14,6 +14,13 @@
 // Prefill portions, decode steps and mixed batches are the same launch, told apart only by the list of runs.  A launch of
 // single tokens (a decode step) may cut each token's keys into num_splits ranges: every range leaves its unnormalised sum,
 // running maximum and running sum in fp32 scratch (the sink belongs to the first range), and a second launch merges them.
+//
+// Averaged blocks (pool > 0, window > 0): beside the window's tokens, token i sees one key / value row for every block b of
+// `pool` positions whose last position precedes its window, b pool + pool - 1 <= i - window; the rows are the means of the
+// block's cached keys and values, kept in pooled buffers at row slot(b pool + pool - 1) / pool_div (mi355_pool_kv_blocks
+// writes them when a block's last token enters the cache).  The walk then starts with the tiles of the pooled rows that the
+// run's last token sees, masked per row, and goes on with the window's tiles; blocks and tokens share the running (max, sum).
+// A gate per head (head_gate, logits) multiplies head h's result by its sigmoid.
 #include "common.cuh"
 
 #include <algorithm>
@@ -37,6 +44,11 @@ struct WaArgs {
   const int64_t* positions;
   const int32_t* blocks;
   const float* sink;
+  const void* pooled_k;
+  const void* pooled_v;
+  const void* gate;        // [token][head] logits of the result's gate, or null
+  int64_t gate_token_stride;
+  int pool, pool_div;
   float* partial;          // num_splits > 1: [split][token][head][dv + 2] = unnormalised result | running max | running sum
   int64_t q_token_stride, q_head_stride, out_token_stride, out_head_stride, req_to_token_stride, tokens;
   int heads, kv_heads, d, dv, heads_per_tile, window, num_splits;
@@ -60,6 +72,8 @@ __device__ __forceinline__ float row16_sum(float x) {
   x += wa_dpp<0x141>(x);
   return x + wa_dpp<0x140>(x);
 }
+
+__device__ __forceinline__ float wa_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 
 // Vector-ALU kernel.  sm: Qs [16][d] | Ks [KT][d + 1] | Vs [KT][dv] | Ps [16][KT]
 template <typename T>
@@ -97,8 +111,12 @@ __global__ __launch_bounds__(256) void window_attention_valu_kernel(WaArgs a) {
   const int lowest = a.window > 0 ? max(0, first - a.window + 1) : 0;
   const int split = blockIdx.z;
   const int all_lo = lowest / WA_KT, all_hi = last / WA_KT + 1;
-  const int per = (all_hi - all_lo + a.num_splits - 1) / a.num_splits;
-  const int tile_lo = all_lo + split * per, tile_hi = min(all_hi, tile_lo + per);
+  // pooled rows that the run's last token sees come first on the walk: ptiles tiles of them, then the window's tiles
+  const int nb_run = (a.pool > 0 && a.window > 0 && last - a.window + 1 >= a.pool) ? (last - a.window + 1) / a.pool : 0;
+  const int ptiles = (nb_run + WA_KT - 1) / WA_KT;
+  const int ntiles = ptiles + all_hi - all_lo;
+  const int per = (ntiles + a.num_splits - 1) / a.num_splits;
+  const int tile_lo = split * per, tile_hi = min(ntiles, tile_lo + per);
   const int r = tid >> 4, cx = tid & 15;
   const int hl_r = r % a.heads_per_tile;
   float run_m = WA_NEG, run_l = 0.f;
@@ -106,20 +124,25 @@ __global__ __launch_bounds__(256) void window_attention_valu_kernel(WaArgs a) {
   float acc[16];
 #pragma unroll
   for (int m = 0; m < 16; ++m) acc[m] = 0.f;
-  const T* kc = (const T*)a.k_cache;
-  const T* vc = (const T*)a.v_cache;
   for (int tile = tile_lo; tile < tile_hi; ++tile) {
-    const int j0 = tile * WA_KT;
+    const bool ptile = tile < ptiles;
+    const int j0 = (ptile ? tile : all_lo + tile - ptiles) * WA_KT;
+    const T* kc = (const T*)(ptile ? a.pooled_k : a.k_cache);
+    const T* vc = (const T*)(ptile ? a.pooled_v : a.v_cache);
     __syncthreads();
-    for (int e = tid; e < WA_KT * d; e += 256) {
-      const int kk = e / d, i = e - kk * d;
+    for (int e = tid; e < WA_KT * (d + dv); e += 256) {
+      const bool isk = e < WA_KT * d;
+      const int e2 = isk ? e : e - WA_KT * d;
+      const int w = isk ? d : dv;
+      const int kk = e2 / w, i = e2 - kk * w;
       const int j = j0 + kk;
-      Ks[kk * (d + 1) + i] = (j >= lowest && j <= last) ? to_f32(kc[((int64_t)table[j] * a.kv_heads + g) * d + i]) : 0.f;
-    }
-    for (int e = tid; e < WA_KT * dv; e += 256) {
-      const int kk = e / dv, i = e - kk * dv;
-      const int j = j0 + kk;
-      Vs[e] = (j >= lowest && j <= last) ? to_f32(vc[((int64_t)table[j] * a.kv_heads + g) * dv + i]) : 0.f;
+      float val = 0.f;
+      if (ptile ? j < nb_run : (j >= lowest && j <= last)) {
+        const int64_t row = ptile ? table[j * a.pool + a.pool - 1] / a.pool_div : table[j];
+        val = to_f32((isk ? kc : vc)[(row * a.kv_heads + g) * w + i]);
+      }
+      if (isk) Ks[kk * (d + 1) + i] = val;
+      else Vs[e2] = val;
     }
     __syncthreads();
     const int rp = row_pos[r];
@@ -131,7 +154,7 @@ __global__ __launch_bounds__(256) void window_attention_valu_kernel(WaArgs a) {
       float s = 0.f;
       for (int i = 0; i < d; ++i) s = fmaf(Qs[r * d + i], Ks[kk * (d + 1) + i], s);
       const int j = j0 + kk;
-      const bool seen = j <= rp && (a.window <= 0 || rp - j < a.window);
+      const bool seen = ptile ? (rp >= 0 && j * a.pool + a.pool - 1 <= rp - a.window) : (j <= rp && (a.window <= 0 || rp - j < a.window));
       sc[u] = seen ? s * a.scale : WA_NEG;
       tmax = fmaxf(tmax, sc[u]);
     }
@@ -172,7 +195,8 @@ __global__ __launch_bounds__(256) void window_attention_valu_kernel(WaArgs a) {
       if (cx == 0) { part[dv] = run_m; part[dv + 1] = run_l; }
       return;
     }
-    const float inv = run_l > 0.f ? 1.0f / run_l : 0.f;
+    float inv = run_l > 0.f ? 1.0f / run_l : 0.f;
+    if (a.gate != nullptr) inv *= wa_sigmoid(to_f32(((const T*)a.gate)[(t0 + tl) * a.gate_token_stride + h0 + hl]));
 #pragma unroll
     for (int m = 0; m < 16; ++m) {
       const int c = cx + 16 * m;
@@ -187,7 +211,8 @@ __global__ __launch_bounds__(256) void window_attention_valu_kernel(WaArgs a) {
 template <typename T>
 __global__ __launch_bounds__(256) void window_attention_merge_kernel(T* __restrict__ out, const float* __restrict__ partial,
                                                                      int64_t tokens, int heads, int dv, int num_splits,
-                                                                     int64_t out_token_stride, int64_t out_head_stride) {
+                                                                     int64_t out_token_stride, int64_t out_head_stride,
+                                                                     const T* __restrict__ gate, int64_t gate_token_stride) {
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int64_t idx = (int64_t)blockIdx.x * 4 + wv;
   if (idx >= tokens * heads) return;
@@ -199,7 +224,8 @@ __global__ __launch_bounds__(256) void window_attention_merge_kernel(T* __restri
   for (int k = 0; k < num_splits; ++k) M = fmaxf(M, p0[k * stride + dv]);
   float L = 0.f;
   for (int k = 0; k < num_splits; ++k) L += p0[k * stride + dv + 1] * expf(p0[k * stride + dv] - M);
-  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  float inv = L > 0.f ? 1.0f / L : 0.f;
+  if (gate != nullptr) inv *= wa_sigmoid(to_f32(gate[t * gate_token_stride + h]));
   for (int c = lane; c < dv; c += 64) {
     float s = 0.f;
     for (int k = 0; k < num_splits; ++k) s += p0[k * stride + c] * expf(p0[k * stride + dv] - M);
@@ -266,8 +292,12 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
   const int lowest = a.window > 0 ? max(0, first - a.window + 1) : 0;
   const int split = blockIdx.z;
   const int all_lo = lowest / WA_KT, all_hi = last / WA_KT + 1;
-  const int per = (all_hi - all_lo + a.num_splits - 1) / a.num_splits;
-  const int tile_lo = all_lo + split * per, tile_hi = min(all_hi, tile_lo + per);
+  // pooled rows that the run's last token sees come first on the walk: ptiles tiles of them, then the window's tiles
+  const int nb_run = (a.pool > 0 && a.window > 0 && last - a.window + 1 >= a.pool) ? (last - a.window + 1) / a.pool : 0;
+  const int ptiles = (nb_run + WA_KT - 1) / WA_KT;
+  const int ntiles = ptiles + all_hi - all_lo;
+  const int per = (ntiles + a.num_splits - 1) / a.num_splits;
+  const int tile_lo = split * per, tile_hi = min(ntiles, tile_lo + per);
   const int nblk = dv / 16;
   // this lane's four score rows: 16 wv + 4 lg + x
   float run_m[4], run_l[4];
@@ -289,15 +319,20 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
   Vec<T, 8> kreg[WAM_MAXC], vreg[WAM_MAXC];
   int64_t ksrc[WAM_MAXC], vsrc[WAM_MAXC];
   // every load is unconditional: chunk numbers past the tile's last one are clamped (and never stored), keys outside
-  // [0, last] are clamped to a valid row (and masked below)
+  // [0, last] (pooled rows past the last one the run sees) are clamped to a valid row (and masked below)
   auto load_slots = [&](int tile) {
-    const int j0 = tile * WA_KT;
+    const bool ptile = tile < ptiles;
+    const int j0 = (ptile ? tile : all_lo + tile - ptiles) * WA_KT;
+    kc = (const T*)(ptile ? a.pooled_k : a.k_cache);
+    vc = (const T*)(ptile ? a.pooled_v : a.v_cache);
 #pragma unroll
     for (int u = 0; u < WAM_MAXC; ++u) {
       const int ek = min(tid + 256 * u, WA_KT * dch - 1), ev = min(tid + 256 * u, WA_KT * vch - 1);
       const int kk = ek / dch, kv = ev / vch;
-      ksrc[u] = ((int64_t)table[min(j0 + kk, last)] * a.kv_heads + g) * d + (ek - kk * dch) * 8;
-      vsrc[u] = ((int64_t)table[min(j0 + kv, last)] * a.kv_heads + g) * dv + (ev - kv * vch) * 8;
+      const int64_t rk = ptile ? table[min(j0 + kk, nb_run - 1) * a.pool + a.pool - 1] / a.pool_div : table[min(j0 + kk, last)];
+      const int64_t rv = ptile ? table[min(j0 + kv, nb_run - 1) * a.pool + a.pool - 1] / a.pool_div : table[min(j0 + kv, last)];
+      ksrc[u] = (rk * a.kv_heads + g) * d + (ek - kk * dch) * 8;
+      vsrc[u] = (rv * a.kv_heads + g) * dv + (ev - kv * vch) * 8;
     }
   };
   auto request = [&]() {
@@ -313,7 +348,8 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
     load_slots(min(tile_lo + 1, tile_hi - 1));
   }
   for (int tile = tile_lo; tile < tile_hi; ++tile) {
-    const int j0 = tile * WA_KT;
+    const bool ptile = tile < ptiles;
+    const int j0 = (ptile ? tile : all_lo + tile - ptiles) * WA_KT;
     __syncthreads();                             // the last tile's readers are done (and, the first time, Qs is written)
 #pragma unroll
     for (int u = 0; u < WAM_MAXC; ++u) {
@@ -347,8 +383,8 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
         const int r = 16 * wv + 4 * lg + x;
         const int rp = row_pos[r];
         const int ja = j0 + li, jb = j0 + 16 + li;
-        const bool va = ja <= rp && (a.window <= 0 || rp - ja < a.window);
-        const bool vb = jb <= rp && (a.window <= 0 || rp - jb < a.window);
+        const bool va = ptile ? (rp >= 0 && ja * a.pool + a.pool - 1 <= rp - a.window) : (ja <= rp && (a.window <= 0 || rp - ja < a.window));
+        const bool vb = ptile ? (rp >= 0 && jb * a.pool + a.pool - 1 <= rp - a.window) : (jb <= rp && (a.window <= 0 || rp - jb < a.window));
         const float sa = va ? s0[x] * a.scale : WA_NEG, sb = vb ? s1[x] * a.scale : WA_NEG;
         const float new_m = fmaxf(run_m[x], row16_max(fmaxf(sa, sb)));
         const float alpha = __expf(run_m[x] - new_m);
@@ -417,9 +453,81 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(WaArgs a) {
           continue;
         }
         const float l = row_l[r];
-        ((T*)a.out)[(t0 + tl) * a.out_token_stride + (int64_t)(h0 + hl) * a.out_head_stride + col] =
-            from_f32<T>(l > 0.f ? acc[rt][c][x] / l : 0.f);
+        float o = l > 0.f ? acc[rt][c][x] / l : 0.f;
+        if (a.gate != nullptr) o *= wa_sigmoid(to_f32(((const T*)a.gate)[(t0 + tl) * a.gate_token_stride + h0 + hl]));
+        ((T*)a.out)[(t0 + tl) * a.out_token_stride + (int64_t)(h0 + hl) * a.out_head_stride + col] = from_f32<T>(o);
       }
+    }
+  }
+}
+
+// One workgroup per token of the step; only a token whose position ends a block of `pool` does anything: it averages the
+// block's cached rows into the pooled buffers' row for the block.  A row is kw key features followed (in another buffer) by
+// vw value features, taken V at a time (16 bytes when the shapes allow, else one); the workgroup's threads form R lanes of
+// rows x C columns of such vectors, lane r sums rows r, r + R, ... in fp32, the lanes' sums meet in LDS in lane order, one
+// multiplication by 1 / pool.  The order of the additions depends on the shapes alone, never on how a prompt was cut.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void pool_kv_blocks_kernel(T* __restrict__ pk, T* __restrict__ pv, const T* __restrict__ kc,
+                                                             const T* __restrict__ vc, const int32_t* __restrict__ req_to_token,
+                                                             const int64_t* __restrict__ req_pool_indices,
+                                                             const int32_t* __restrict__ tok_req,
+                                                             const int64_t* __restrict__ positions, int64_t req_to_token_stride,
+                                                             int kw, int vw, int pool, int pool_div) {
+  __shared__ float part[256 * V];
+  const int64_t t = blockIdx.x;
+  const int pos = (int)positions[t];
+  if ((pos + 1) % pool != 0) return;
+  const int b = tok_req != nullptr ? tok_req[t] : (int)t;
+  const int32_t* table = req_to_token + req_pool_indices[b] * req_to_token_stride + (pos - pool + 1);
+  const int64_t dst = table[pool - 1] / pool_div;
+  const float inv = 1.0f / (float)pool;
+  const int nk = kw / V, nv = (kw + vw) / V;           // vectors per row: keys first, then values
+  const int C = min(nv, 256);                          // columns handled at a time
+  int R = 256 / C;                                     // lanes of rows
+  R = min(R, pool);
+  const int tid = threadIdx.x;
+  const int col = tid % C, lane = tid / C;
+  for (int c0 = 0; c0 < nv; c0 += C) {
+    const int c = c0 + col;
+    const bool live = lane < R && c < nv;
+    const bool isk = c < nk;
+    const T* src = isk ? kc : vc;
+    const int w = isk ? kw : vw;
+    const int off = (isk ? c : c - nk) * V;
+    float acc[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) acc[k] = 0.f;
+    if (live) {
+      int j = lane;
+      for (; j + 3 * R < pool; j += 4 * R) {           // four rows in flight
+        const Vec<T, V> a0 = ldvec<T, V>(src + (int64_t)table[j] * w + off);
+        const Vec<T, V> a1 = ldvec<T, V>(src + (int64_t)table[j + R] * w + off);
+        const Vec<T, V> a2 = ldvec<T, V>(src + (int64_t)table[j + 2 * R] * w + off);
+        const Vec<T, V> a3 = ldvec<T, V>(src + (int64_t)table[j + 3 * R] * w + off);
+#pragma unroll
+        for (int k = 0; k < V; ++k) acc[k] = ((acc[k] + to_f32(a0.v[k])) + to_f32(a1.v[k])) + (to_f32(a2.v[k]) + to_f32(a3.v[k]));
+      }
+      for (; j < pool; j += R) {
+        const Vec<T, V> a0 = ldvec<T, V>(src + (int64_t)table[j] * w + off);
+#pragma unroll
+        for (int k = 0; k < V; ++k) acc[k] += to_f32(a0.v[k]);
+      }
+    }
+    __syncthreads();                                   // the last pass's readers are done
+    if (live) {
+#pragma unroll
+      for (int k = 0; k < V; ++k) part[(lane * C + col) * V + k] = acc[k];
+    }
+    __syncthreads();
+    if (live && lane == 0) {
+      Vec<T, V> out;
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        float sum = part[col * V + k];
+        for (int r = 1; r < R; ++r) sum += part[(r * C + col) * V + k];
+        out.v[k] = from_f32<T>(sum * inv);
+      }
+      stvec<T, V>((isk ? pk : pv) + dst * w + off, out);
     }
   }
 }
@@ -477,6 +585,23 @@ int mi355_window_attention(void* out, const void* q, const void* k_cache, const 
                            int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t req_to_token_stride,
                            int heads, int kv_heads, int head_dim, int v_head_dim, int window, float scale, int num_splits,
                            float* split_scratch, int64_t tokens, int max_run, int dtype, void* stream) {
+  return mi355_window_attention_pooled(out, q, k_cache, v_cache, nullptr, nullptr, req_to_token, req_pool_indices, tok_req, positions,
+                                       blocks, num_blocks, sink, nullptr, 0, q_token_stride, q_head_stride, out_token_stride,
+                                       out_head_stride, req_to_token_stride, heads, kv_heads, head_dim, v_head_dim, window, 0, 1,
+                                       scale, num_splits, split_scratch, tokens, max_run, dtype, stream);
+}
+
+int mi355_window_attention_pooled(void* out, const void* q, const void* k_cache, const void* v_cache, const void* pooled_k,
+                                  const void* pooled_v, const int32_t* req_to_token, const int64_t* req_pool_indices,
+                                  const int32_t* tok_req, const int64_t* positions, const int32_t* blocks, int64_t num_blocks,
+                                  const float* sink, const void* head_gate, int64_t gate_token_stride, int64_t q_token_stride,
+                                  int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride,
+                                  int64_t req_to_token_stride, int heads, int kv_heads, int head_dim, int v_head_dim, int window,
+                                  int pool, int pool_div, float scale, int num_splits, float* split_scratch, int64_t tokens,
+                                  int max_run, int dtype, void* stream) {
+  MI355_REQUIRE(pool >= 0 && pool_div >= 1 && (pool == 0 || (pooled_k && pooled_v && window > 0)), MI355_ERR_INVALID,
+                "window_attention: averaged blocks need their buffers and a window");
+  MI355_REQUIRE(head_gate == nullptr || gate_token_stride >= heads, MI355_ERR_INVALID, "window_attention: bad gate stride");
   MI355_REQUIRE(num_splits >= 1 && num_splits <= 64 && (num_splits == 1 || (split_scratch && blocks == nullptr)), MI355_ERR_INVALID,
                 "window_attention: key splits serve launches of one token per run and need scratch");
   MI355_REQUIRE(out && q && k_cache && v_cache && req_to_token && req_pool_indices && positions, MI355_ERR_INVALID,
@@ -490,12 +615,14 @@ int mi355_window_attention(void* out, const void* q, const void* k_cache, const 
   WaArgs a;
   a.out = out; a.q = q; a.k_cache = k_cache; a.v_cache = v_cache; a.req_to_token = req_to_token;
   a.req_pool_indices = req_pool_indices; a.tok_req = tok_req; a.positions = positions; a.blocks = blocks; a.sink = sink;
+  a.pooled_k = pooled_k; a.pooled_v = pooled_v; a.gate = head_gate; a.gate_token_stride = gate_token_stride; a.pool = pool;
+  a.pool_div = pool_div;
   a.q_token_stride = q_token_stride; a.q_head_stride = q_head_stride; a.out_token_stride = out_token_stride;
   a.out_head_stride = out_head_stride; a.req_to_token_stride = req_to_token_stride; a.tokens = tokens; a.heads = heads;
   // the matrix-core kernel needs 16-byte rows everywhere; a caller whose q is laid out otherwise gets the vector-ALU kernel,
   // whose runs are shorter: max_run says how long the caller's runs may be, and a launch that cannot take them is refused
   const bool mfma = wa_mfma_shape(dtype, head_dim, v_head_dim) && q_token_stride % 8 == 0 && q_head_stride % 8 == 0 &&
-                    aligned16(q) && aligned16(k_cache) && aligned16(v_cache);
+                    aligned16(q) && aligned16(k_cache) && aligned16(v_cache) && (pool == 0 || (aligned16(pooled_k) && aligned16(pooled_v)));
   const int rows = mfma ? WAM_ROWS : WA_ROWS;
   a.kv_heads = kv_heads; a.d = head_dim; a.dv = v_head_dim; a.heads_per_tile = wa_heads_per_tile(heads, kv_heads, rows);
   a.window = window; a.scale = scale; a.num_splits = num_splits; a.partial = split_scratch;
@@ -514,9 +641,36 @@ int mi355_window_attention(void* out, const void* q, const void* k_cache, const 
     const unsigned g2 = (unsigned)((tokens * heads + 3) / 4);
     MI355_DISPATCH_DTYPE(dtype, "window_attention", {
       hipLaunchKernelGGL((window_attention_merge_kernel<T>), dim3(g2), dim3(256), 0, (hipStream_t)stream, (T*)out, split_scratch, tokens,
-                         heads, v_head_dim, num_splits, out_token_stride, out_head_stride);
+                         heads, v_head_dim, num_splits, out_token_stride, out_head_stride, (const T*)head_gate, gate_token_stride);
     });
     MI355_CHECK_LAUNCH("window_attention(merge)");
   }
+  return MI355_OK;
+}
+
+int mi355_pool_kv_blocks(void* pooled_k, void* pooled_v, const void* k_cache, const void* v_cache, const int32_t* req_to_token,
+                         const int64_t* req_pool_indices, const int32_t* tok_req, const int64_t* positions, int64_t tokens,
+                         int64_t req_to_token_stride, int kv_heads, int head_dim, int v_head_dim, int pool, int pool_div, int dtype,
+                         void* stream) {
+  MI355_REQUIRE(pooled_k && pooled_v && k_cache && v_cache && req_to_token && req_pool_indices && positions, MI355_ERR_INVALID,
+                "pool_kv_blocks: null pointer");
+  MI355_REQUIRE(tokens >= 0 && tokens <= 0x7fffffff && kv_heads > 0 && head_dim > 0 && v_head_dim > 0 && pool >= 1 && pool_div >= 1,
+                MI355_ERR_INVALID, "pool_kv_blocks: bad shape");
+  if (tokens == 0) return MI355_OK;
+  const int kw = kv_heads * head_dim, vw = kv_heads * v_head_dim;
+  const int vecw = dtype == MI355_F32 ? 4 : 8;
+  const bool vec = kw % vecw == 0 && vw % vecw == 0 && aligned16(pooled_k) && aligned16(pooled_v) && aligned16(k_cache) && aligned16(v_cache);
+  MI355_DISPATCH_DTYPE(dtype, "pool_kv_blocks", {
+    constexpr int V = 16 / sizeof(T);
+    if (vec)
+      hipLaunchKernelGGL((pool_kv_blocks_kernel<T, V>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (T*)pooled_k,
+                         (T*)pooled_v, (const T*)k_cache, (const T*)v_cache, req_to_token, req_pool_indices, tok_req, positions,
+                         req_to_token_stride, kw, vw, pool, pool_div);
+    else
+      hipLaunchKernelGGL((pool_kv_blocks_kernel<T, 1>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (T*)pooled_k,
+                         (T*)pooled_v, (const T*)k_cache, (const T*)v_cache, req_to_token, req_pool_indices, tok_req, positions,
+                         req_to_token_stride, kw, vw, pool, pool_div);
+  });
+  MI355_CHECK_LAUNCH("pool_kv_blocks");
   return MI355_OK;
 }

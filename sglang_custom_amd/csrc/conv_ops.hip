@@ -1,5 +1,5 @@
 // Short causal convolutions over time, one filter per channel, for sequences that arrive in pieces:
-//     y[t][c] = act( (residual ? u[t][c] : 0) + sum_{k < taps} w[c][taps - 1 - k] * u[t - k][c] ),   u = 0 before position 0
+//     y[t][c] = act( (residual ? u[t][c] : 0) + sum_{k < taps} w[c][taps - 1 - k] * u[t - k][c] [+ bias[c]] ),   u = 0 before position 0
 // The last taps - 1 inputs of a sequence are its state (fp32 rows [slots, taps - 1, C], row taps - 2 the most recent): a
 // step's first tokens read them, and after the step they are replaced by the step's own last inputs.
 //   * mi355_causal_conv: every (token, channel) in one launch; up to two filters read the same input (two outputs).  In a
@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(T* __restrict__ y1, T*
                                                           const int64_t* __restrict__ req_pool_indices,
                                                           const int32_t* __restrict__ tok_req, const int32_t* __restrict__ seg_start,
                                                           const int64_t* __restrict__ positions, int64_t C, int taps, int residual,
-                                                          int act) {
+                                                          int act, const T* __restrict__ bias) {
   const int64_t t = blockIdx.x;
   const int64_t c = (int64_t)blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
@@ -57,6 +57,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(T* __restrict__ y1, T*
     if (w2 != nullptr) a2 = fmaf(to_f32(w2[c * taps + (taps - 1 - k)]), in[k], a2);
   }
   if (residual) { a1 += in[0]; a2 += in[0]; }
+  if (bias != nullptr) a1 += to_f32(bias[c]);
   y1[t * C + c] = from_f32<T>(conv_act(a1, act));
   if (w2 != nullptr) y2[t * C + c] = from_f32<T>(conv_act(a2, act));
   if (tok_req == nullptr) {
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(256) void causal_conv_vec_kernel(T* __restrict__ y1
                                                               const int64_t* __restrict__ req_pool_indices,
                                                               const int32_t* __restrict__ tok_req, const int32_t* __restrict__ seg_start,
                                                               const int64_t* __restrict__ positions, int64_t tokens, int64_t C,
-                                                              int residual, int act) {
+                                                              int residual, int act, const T* __restrict__ bias) {
   const int64_t groups = C / V;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t tb = idx / groups;
@@ -100,6 +101,15 @@ __global__ __launch_bounds__(256) void causal_conv_vec_kernel(T* __restrict__ y1
 #pragma unroll
       for (int v = 0; v < V; ++v) wf[f][i * V + v] = to_f32(x.v[v]);
     }
+  }
+  float bf[V];                                       // the first filter's bias
+  if (bias != nullptr) {
+    const Vec<T, V> x = ldvec<T, V>(bias + c);
+#pragma unroll
+    for (int v = 0; v < V; ++v) bf[v] = to_f32(x.v[v]);
+  } else {
+#pragma unroll
+    for (int v = 0; v < V; ++v) bf[v] = 0.f;
   }
   float in[TAPS][V];                                 // in[k]: the input k tokens back
 #pragma unroll
@@ -150,6 +160,7 @@ __global__ __launch_bounds__(256) void causal_conv_vec_kernel(T* __restrict__ y1
 #pragma unroll
         for (int k = TAPS - 1; k >= 0; --k) a = fmaf(wf[f][v * TAPS + (TAPS - 1 - k)], in[k][v], a);     // oldest tap first
         if (residual) a += in[0][v];
+        if (f == 0) a += bf[v];
         out.v[v] = from_f32<T>(conv_act(a, act));
       }
       stvec<T, V>((f == 0 ? y1 : y2) + t * C + c, out);
@@ -169,12 +180,12 @@ __global__ __launch_bounds__(256) void causal_conv_vec_kernel(T* __restrict__ y1
 template <typename T, int TAPS>
 void launch_conv_vec(void* y1, void* y2, const void* u, int64_t u_stride, const void* w1, const void* w2, float* state,
                      const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* tok_req, const int32_t* seg_start,
-                     const int64_t* positions, int64_t tokens, int64_t channels, int residual, int act, hipStream_t stream) {
+                     const int64_t* positions, int64_t tokens, int64_t channels, int residual, int act, const void* bias, hipStream_t stream) {
   constexpr int V = 16 / sizeof(T);
   const int64_t n = ((tokens + CONV_TT - 1) / CONV_TT) * (channels / V);
   hipLaunchKernelGGL((causal_conv_vec_kernel<T, V, TAPS>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, (T*)y1, (T*)y2,
                      (const T*)u, u_stride, (const T*)w1, (const T*)w2, state, req_to_state, req_pool_indices, tok_req, seg_start,
-                     positions, tokens, channels, residual, act);
+                     positions, tokens, channels, residual, act, (const T*)bias);
 }
 
 template <typename T>
@@ -222,6 +233,14 @@ int mi355_causal_conv(void* y1, void* y2, const void* u, int64_t u_stride, const
                       const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* tok_req,
                       const int32_t* seg_start, const int64_t* positions, int64_t tokens, int64_t channels, int taps,
                       int residual, int act, int dtype, void* stream) {
+  return mi355_causal_conv_bias(y1, y2, u, u_stride, w1, w2, nullptr, state, req_to_state, req_pool_indices, tok_req, seg_start,
+                                positions, tokens, channels, taps, residual, act, dtype, stream);
+}
+
+int mi355_causal_conv_bias(void* y1, void* y2, const void* u, int64_t u_stride, const void* w1, const void* w2, const void* bias1,
+                           float* state, const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* tok_req,
+                           const int32_t* seg_start, const int64_t* positions, int64_t tokens, int64_t channels, int taps,
+                           int residual, int act, int dtype, void* stream) {
   MI355_REQUIRE(y1 && u && w1 && (state || taps == 1) && req_to_state && req_pool_indices && positions, MI355_ERR_INVALID, "causal_conv: null pointer");
   MI355_REQUIRE((w2 == nullptr) == (y2 == nullptr), MI355_ERR_INVALID, "causal_conv: the second filter comes with its output");
   MI355_REQUIRE((tok_req == nullptr) == (seg_start == nullptr), MI355_ERR_INVALID, "causal_conv: tok_req and seg_start come together");
@@ -232,13 +251,14 @@ int mi355_causal_conv(void* y1, void* y2, const void* u, int64_t u_stride, const
   const int esz = dtype == MI355_F32 ? 4 : 2, vw = 16 / esz;
   const bool vec = channels % vw == 0 && u_stride % vw == 0 && aligned16(u) && aligned16(y1) && aligned16(w1) &&
                    (y2 == nullptr || (aligned16(y2) && aligned16(w2))) && (taps == 1 || aligned16(state)) && channels % 4 == 0 &&
+                   (bias1 == nullptr || aligned16(bias1)) &&
                    tokens * (channels / vw) < ((int64_t)1 << 31) * 256;
   if (vec) {
 #define MI355_CONV_TAPS(N)                                                                                                    \
   case N:                                                                                                                     \
     MI355_DISPATCH_DTYPE(dtype, "causal_conv", {                                                                              \
       launch_conv_vec<T, N>(y1, y2, u, u_stride, w1, w2, state, req_to_state, req_pool_indices, tok_req, seg_start, positions,   \
-                            tokens, channels, residual, act, (hipStream_t)stream);                                            \
+                            tokens, channels, residual, act, bias1, (hipStream_t)stream);                                     \
     });                                                                                                                       \
     break;
     switch (taps) {
@@ -254,7 +274,7 @@ int mi355_causal_conv(void* y1, void* y2, const void* u, int64_t u_stride, const
   MI355_DISPATCH_DTYPE(dtype, "causal_conv", {
     hipLaunchKernelGGL((causal_conv_kernel<T>), grid, dim3(256), 0, (hipStream_t)stream, (T*)y1, (T*)y2, (const T*)u, u_stride,
                        (const T*)w1, (const T*)w2, state, req_to_state, req_pool_indices, tok_req, seg_start, positions, channels,
-                       taps, residual, act);
+                       taps, residual, act, (const T*)bias1);
   });
   MI355_CHECK_LAUNCH("causal_conv");
   return MI355_OK;

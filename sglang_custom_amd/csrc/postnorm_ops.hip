@@ -112,24 +112,52 @@ __global__ __launch_bounds__(256) void scaled_add_group_rmsnorm_kernel(
   }
 }
 
-// One workgroup per token: x[t] += y[t] / sqrt(mean(y[t]^2) + eps) * w
-template <typename T>
+// One workgroup per token: x[t] += mult * ls * y[t] / sqrt(mean(y[t]^2) + eps) * (offset + w)   (ls null: ones).  VEC: eight
+// features per access (16-byte loads of y, w and ls, two 16-byte loads and stores of the fp32 row, 16-byte stores of the
+// copy); the second pass over y finds it in the cache.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void rmsnorm_residual_add_kernel(float* __restrict__ x, T* __restrict__ h_out,
                                                                    const T* __restrict__ y, int64_t y_stride,
-                                                                   const T* __restrict__ w, int64_t D, float eps) {
+                                                                   const T* __restrict__ w, const T* __restrict__ ls, float offset,
+                                                                   float mult, int64_t D, float eps) {
   __shared__ float red[16];
+  constexpr int W = VEC ? 8 : 1;
   const int64_t t = blockIdx.x;
   float q = 0.f;
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-    const float v = to_f32(y[t * y_stride + i]);
-    q += v * v;
+  for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+    const Vec<T, W> v = ldvec<T, W>(y + t * y_stride + i);
+#pragma unroll
+    for (int k = 0; k < W; ++k) q += to_f32(v.v[k]) * to_f32(v.v[k]);
   }
   q = block_sum(q, red);
   const float inv = 1.0f / sqrtf(q / (float)D + eps);
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-    const float v = x[t * D + i] + to_f32(y[t * y_stride + i]) * inv * to_f32(w[i]);
-    x[t * D + i] = v;
-    if (h_out != nullptr) h_out[t * D + i] = from_f32<T>(v);
+  for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+    const Vec<T, W> v = ldvec<T, W>(y + t * y_stride + i);
+    const Vec<T, W> wv = ldvec<T, W>(w + i);
+    Vec<T, W> lv;
+    if (ls != nullptr) lv = ldvec<T, W>(ls + i);
+    float r[W];
+    if constexpr (VEC) {
+      const float4 a = *reinterpret_cast<const float4*>(x + t * D + i), b = *reinterpret_cast<const float4*>(x + t * D + i + 4);
+      r[0] = a.x; r[1] = a.y; r[2] = a.z; r[3] = a.w; r[4] = b.x; r[5] = b.y; r[6] = b.z; r[7] = b.w;
+    } else {
+      r[0] = x[t * D + i];
+    }
+    Vec<T, W> hv;
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      float n = to_f32(v.v[k]) * inv * (offset + to_f32(wv.v[k]));
+      if (ls != nullptr) n *= to_f32(lv.v[k]);
+      r[k] += mult * n;
+      hv.v[k] = from_f32<T>(r[k]);
+    }
+    if constexpr (VEC) {
+      *reinterpret_cast<float4*>(x + t * D + i) = make_float4(r[0], r[1], r[2], r[3]);
+      *reinterpret_cast<float4*>(x + t * D + i + 4) = make_float4(r[4], r[5], r[6], r[7]);
+    } else {
+      x[t * D + i] = r[0];
+    }
+    if (h_out != nullptr) stvec<T, W>(h_out + t * D + i, hv);
   }
 }
 
@@ -139,7 +167,7 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(
     OT* __restrict__ out, const T* __restrict__ src, const T* __restrict__ w, const int64_t* __restrict__ positions,
     const int64_t* __restrict__ loc, const float* __restrict__ inv_freq, int64_t tokens, int heads, int d, int64_t src_token_stride,
     int64_t src_head_stride, int64_t out_token_stride, int64_t out_head_stride, int rot_dims, int interleaved, float scale,
-    float eps) {
+    float eps, float rot_mag) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int64_t idx = (int64_t)blockIdx.x * 4 + wv;
@@ -184,10 +212,131 @@ __global__ __launch_bounds__(256) void head_norm_rope_kernel(
       const float u = row[partner] * inv * (w != nullptr ? to_f32(w[partner]) : 1.0f);
       float sn, cs;
       sincosf(pos * inv_freq[pair], &sn, &cs);
+      sn *= rot_mag;
+      cs *= rot_mag;
       // (a, b) -> (a cos - b sin, b cos + a sin): v is a for the first of the pair, b for the second
       v = second ? v * cs + u * sn : v * cs - u * sn;
     }
     o[i] = from_f32<OT>(v * scale);
+  }
+}
+
+// The three head norms of an attention layer in one launch.  One wave per (token, unit), unit = a query head (RMS norm with
+// wq, rotation, to q_out [tokens, heads, d]), a key head (RMS norm with wk, rotation, into k_cache[loc[t]]) or a value head
+// (division by its root mean square alone, into v_cache[loc[t]]); the arithmetic per row is head_norm_rope_kernel's.
+// sm: 4 rows of max(d, dv) floats.
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_norm_rope_write_kernel(
+    T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, const T* __restrict__ q, const T* __restrict__ k,
+    const T* __restrict__ v, int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, const T* __restrict__ wq,
+    const T* __restrict__ wk, const int64_t* __restrict__ positions, const int64_t* __restrict__ loc,
+    const float* __restrict__ inv_freq, int64_t tokens, int heads, int kv_heads, int d, int dv, int rot_dims, int interleaved,
+    float eps, float rot_mag) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int units = heads + 2 * kv_heads;
+  const int64_t idx = (int64_t)blockIdx.x * 4 + wv;
+  const bool valid = idx < tokens * units;
+  const int64_t t = valid ? idx / units : 0;
+  const int u = valid ? (int)(idx - t * units) : 0;
+  const T* s;
+  const T* w;
+  T* o;
+  int width, rot;
+  if (u < heads) {
+    s = q + t * q_token_stride + (int64_t)u * d; w = wq; width = d; rot = rot_dims;
+    o = q_out + (t * heads + u) * (int64_t)d;
+  } else if (u < heads + kv_heads) {
+    const int g = u - heads;
+    s = k + t * k_token_stride + (int64_t)g * d; w = wk; width = d; rot = rot_dims;
+    o = k_cache + (loc[t] * kv_heads + g) * (int64_t)d;
+  } else {
+    const int g = u - heads - kv_heads;
+    s = v + t * v_token_stride + (int64_t)g * dv; w = nullptr; width = dv; rot = 0;
+    o = v_cache + (loc[t] * kv_heads + g) * (int64_t)dv;
+  }
+  float* row = sm + (int64_t)wv * max(d, dv);
+  float qs = 0.f;
+  if (valid) {
+    for (int i = lane; i < width; i += 64) {
+      const float x = to_f32(s[i]);
+      row[i] = x;
+      qs += x * x;
+    }
+  }
+  qs = wave_sum(qs);
+  const float inv = 1.0f / sqrtf(qs / (float)width + eps);
+  __syncthreads();
+  if (!valid) return;
+  const float pos = (float)positions[t];
+  const int half = rot / 2;
+  for (int i = lane; i < width; i += 64) {
+    float x = row[i] * inv * (w != nullptr ? to_f32(w[i]) : 1.0f);
+    if (i < rot) {
+      int pair, partner;
+      bool second;
+      if (interleaved) {
+        pair = i >> 1;
+        second = (i & 1) != 0;
+        partner = i ^ 1;
+      } else {
+        second = i >= half;
+        pair = second ? i - half : i;
+        partner = second ? i - half : i + half;
+      }
+      const float y = row[partner] * inv * (w != nullptr ? to_f32(w[partner]) : 1.0f);
+      float sn, cs;
+      sincosf(pos * inv_freq[pair], &sn, &cs);
+      sn *= rot_mag;
+      cs *= rot_mag;
+      x = second ? x * cs + y * sn : x * cs - y * sn;
+    }
+    o[i] = from_f32<T>(x);
+  }
+}
+
+// One workgroup per (token, part): out = N(y * silu(gate)) * w over one of `groups` equal consecutive parts of the row, the
+// gate applied BEFORE the norm.  y fp32 [tokens, D] contiguous, gate T row-strided, w T [D].  A part of up to 2048 features
+// keeps its gated values in registers between the two passes.
+constexpr int GGN_KEEP = 8;
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(T* __restrict__ out, const float* __restrict__ y,
+                                                                  const T* __restrict__ gate, int64_t gate_stride,
+                                                                  const T* __restrict__ w, int64_t D, int groups, float eps) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x / groups;
+  const int part = (int)(blockIdx.x - t * groups);
+  const int64_t n = D / groups, c0 = (int64_t)part * n;
+  const float* yr = y + t * D + c0;
+  const T* gr = gate + t * gate_stride + c0;
+  float keep[GGN_KEEP];
+  float q = 0.f;
+#pragma unroll
+  for (int u = 0; u < GGN_KEEP; ++u) {
+    const int64_t i = threadIdx.x + 256 * u;
+    float v = 0.f;
+    if (i < n) {
+      const float z = to_f32(gr[i]);
+      v = yr[i] * (z * pn_sigmoid(z));
+    }
+    keep[u] = v;
+    q += v * v;
+  }
+  for (int64_t i = threadIdx.x + 256 * GGN_KEEP; i < n; i += 256) {
+    const float z = to_f32(gr[i]);
+    const float v = yr[i] * (z * pn_sigmoid(z));
+    q += v * v;
+  }
+  q = block_sum(q, red);
+  const float inv = 1.0f / sqrtf(q / (float)n + eps);
+#pragma unroll
+  for (int u = 0; u < GGN_KEEP; ++u) {
+    const int64_t i = threadIdx.x + 256 * u;
+    if (i < n) out[t * D + c0 + i] = from_f32<T>(keep[u] * inv * to_f32(w[c0 + i]));
+  }
+  for (int64_t i = threadIdx.x + 256 * GGN_KEEP; i < n; i += 256) {
+    const float z = to_f32(gr[i]);
+    out[t * D + c0 + i] = from_f32<T>(yr[i] * (z * pn_sigmoid(z)) * inv * to_f32(w[c0 + i]));
   }
 }
 
@@ -390,12 +539,25 @@ int mi355_scaled_add_group_rmsnorm(float* x_out, void* h_out, const float* x, co
 
 int mi355_rmsnorm_residual_add(float* x, void* h_out, const void* y, int64_t y_stride, const void* weight, int64_t tokens,
                                int64_t hidden, float eps, int dtype, void* stream) {
+  return mi355_rmsnorm_residual_add_scaled(x, h_out, y, y_stride, weight, nullptr, 0.f, 1.f, tokens, hidden, eps, dtype, stream);
+}
+
+int mi355_rmsnorm_residual_add_scaled(float* x, void* h_out, const void* y, int64_t y_stride, const void* weight,
+                                      const void* layer_scale, float offset, float mult, int64_t tokens, int64_t hidden, float eps,
+                                      int dtype, void* stream) {
   MI355_REQUIRE(x && y && weight, MI355_ERR_INVALID, "rmsnorm_residual_add: null pointer");
   MI355_REQUIRE(tokens >= 0 && hidden > 0 && y_stride >= hidden, MI355_ERR_INVALID, "rmsnorm_residual_add: bad shape");
   if (tokens == 0) return MI355_OK;
+  // eight 16-bit features are one 16-byte access; fp32 activations (four to 16 bytes) take the scalar kernel
+  const bool vec = dtype != MI355_F32 && hidden % 8 == 0 && y_stride % 8 == 0 && aligned16(x) && aligned16(y) && aligned16(weight) &&
+                   (h_out == nullptr || aligned16(h_out)) && (layer_scale == nullptr || aligned16(layer_scale));
   MI355_DISPATCH_DTYPE(dtype, "rmsnorm_residual_add", {
-    hipLaunchKernelGGL((rmsnorm_residual_add_kernel<T>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x, (T*)h_out,
-                       (const T*)y, y_stride, (const T*)weight, hidden, eps);
+    if (vec)
+      hipLaunchKernelGGL((rmsnorm_residual_add_kernel<T, true>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x, (T*)h_out,
+                         (const T*)y, y_stride, (const T*)weight, (const T*)layer_scale, offset, mult, hidden, eps);
+    else
+      hipLaunchKernelGGL((rmsnorm_residual_add_kernel<T, false>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x, (T*)h_out,
+                         (const T*)y, y_stride, (const T*)weight, (const T*)layer_scale, offset, mult, hidden, eps);
   });
   MI355_CHECK_LAUNCH("rmsnorm_residual_add");
   return MI355_OK;
@@ -405,6 +567,16 @@ int mi355_head_norm_rope(void* out, const void* src, const void* weight, const i
                          const float* inv_freq, int64_t tokens, int heads, int head_dim, int64_t src_token_stride,
                          int64_t src_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t out_rows, int rot_dims,
                          int interleaved, float scale, float eps, int dtype, int out_dtype, void* stream) {
+  return mi355_head_norm_rope_mag(out, src, weight, positions, loc, inv_freq, tokens, heads, head_dim, src_token_stride,
+                                  src_head_stride, out_token_stride, out_head_stride, out_rows, rot_dims, interleaved, scale, eps,
+                                  1.0f, dtype, out_dtype, stream);
+}
+
+int mi355_head_norm_rope_mag(void* out, const void* src, const void* weight, const int64_t* positions, const int64_t* loc,
+                             const float* inv_freq, int64_t tokens, int heads, int head_dim, int64_t src_token_stride,
+                             int64_t src_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t out_rows,
+                             int rot_dims, int interleaved, float scale, float eps, float rot_mag, int dtype, int out_dtype,
+                             void* stream) {
   MI355_REQUIRE(out && src && positions, MI355_ERR_INVALID, "head_norm_rope: null pointer");
   MI355_REQUIRE(tokens >= 0 && heads > 0 && head_dim > 0 && head_dim <= 4096 && out_rows >= 0, MI355_ERR_INVALID,
                 "head_norm_rope: bad shape");
@@ -419,11 +591,11 @@ int mi355_head_norm_rope(void* out, const void* src, const void* weight, const i
     if (out_dtype == dtype) {
       hipLaunchKernelGGL((head_norm_rope_kernel<T, T>), dim3(grid), dim3(256), lds, (hipStream_t)stream, (T*)out, (const T*)src,
                          (const T*)weight, positions, loc, inv_freq, tokens, heads, head_dim, src_token_stride, src_head_stride,
-                         out_token_stride, out_head_stride, rot_dims, interleaved, scale, eps);
+                         out_token_stride, out_head_stride, rot_dims, interleaved, scale, eps, rot_mag);
     } else {
       hipLaunchKernelGGL((head_norm_rope_kernel<T, float>), dim3(grid), dim3(256), lds, (hipStream_t)stream, (float*)out,
                          (const T*)src, (const T*)weight, positions, loc, inv_freq, tokens, heads, head_dim, src_token_stride,
-                         src_head_stride, out_token_stride, out_head_stride, rot_dims, interleaved, scale, eps);
+                         src_head_stride, out_token_stride, out_head_stride, rot_dims, interleaved, scale, eps, rot_mag);
     }
   });
   MI355_CHECK_LAUNCH("head_norm_rope");
@@ -448,6 +620,44 @@ int mi355_head_rmsnorm_gate_act(void* out, const float* o, const void* weight, c
                        (const T*)gate, gate_stride, tokens, heads, value_dim, eps, gate_act);
   });
   MI355_CHECK_LAUNCH("head_rmsnorm_gate");
+  return MI355_OK;
+}
+
+int mi355_qkv_norm_rope_write(void* q_out, void* k_cache, void* v_cache, const void* q, const void* k, const void* v,
+                              int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, const void* wq, const void* wk,
+                              const int64_t* positions, const int64_t* loc, const float* inv_freq, int64_t tokens, int heads,
+                              int kv_heads, int head_dim, int v_head_dim, int rot_dims, int interleaved, float eps, float rot_mag,
+                              int dtype, void* stream) {
+  MI355_REQUIRE(q_out && k_cache && v_cache && q && k && v && wq && wk && positions && loc, MI355_ERR_INVALID,
+                "qkv_norm_rope_write: null pointer");
+  MI355_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && head_dim <= 4096 && v_head_dim > 0 && v_head_dim <= 4096,
+                MI355_ERR_INVALID, "qkv_norm_rope_write: bad shape");
+  MI355_REQUIRE(rot_dims >= 0 && rot_dims <= head_dim && rot_dims % 2 == 0 && (rot_dims == 0 || inv_freq), MI355_ERR_INVALID,
+                "qkv_norm_rope_write: rot_dims must be even, at most head_dim, and come with frequencies");
+  if (tokens == 0) return MI355_OK;
+  const size_t lds = (size_t)4 * std::max(head_dim, v_head_dim) * sizeof(float);
+  const unsigned grid = (unsigned)((tokens * (heads + 2 * kv_heads) + 3) / 4);
+  MI355_DISPATCH_DTYPE(dtype, "qkv_norm_rope_write", {
+    hipLaunchKernelGGL((qkv_norm_rope_write_kernel<T>), dim3(grid), dim3(256), lds, (hipStream_t)stream, (T*)q_out, (T*)k_cache,
+                       (T*)v_cache, (const T*)q, (const T*)k, (const T*)v, q_token_stride, k_token_stride, v_token_stride, (const T*)wq,
+                       (const T*)wk, positions, loc, inv_freq, tokens, heads, kv_heads, head_dim, v_head_dim, rot_dims, interleaved, eps,
+                       rot_mag);
+  });
+  MI355_CHECK_LAUNCH("qkv_norm_rope_write");
+  return MI355_OK;
+}
+
+int mi355_gated_group_rmsnorm(void* out, const float* y, const void* gate, int64_t gate_stride, const void* weight, int64_t tokens,
+                              int64_t hidden, int groups, float eps, int dtype, void* stream) {
+  MI355_REQUIRE(out && y && gate && weight, MI355_ERR_INVALID, "gated_group_rmsnorm: null pointer");
+  MI355_REQUIRE(tokens >= 0 && hidden > 0 && groups >= 1 && hidden % groups == 0 && gate_stride >= hidden &&
+                    tokens * groups < ((int64_t)1 << 31), MI355_ERR_INVALID, "gated_group_rmsnorm: bad shape");
+  if (tokens == 0) return MI355_OK;
+  MI355_DISPATCH_DTYPE(dtype, "gated_group_rmsnorm", {
+    hipLaunchKernelGGL((gated_group_rmsnorm_kernel<T>), dim3((unsigned)(tokens * groups)), dim3(256), 0, (hipStream_t)stream, (T*)out, y,
+                       (const T*)gate, gate_stride, (const T*)weight, hidden, groups, eps);
+  });
+  MI355_CHECK_LAUNCH("gated_group_rmsnorm");
   return MI355_OK;
 }
 

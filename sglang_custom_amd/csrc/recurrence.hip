@@ -1,7 +1,10 @@
 // Linear recurrences with one fp32 matrix per (sequence, head); the plain one:
 //     S_t = diag(a_t) S_{t-1} + k_t v_t^T        S [dk, dv]
 //     o_t = S_t^T (q_t * q_scale)
-// a_t either per key channel and token, a = exp(logsigmoid(z + b) / tau) from gate logits z (fp32), or one number per head.
+// a_t either per key channel and token, a = exp(logsigmoid(z + b) / tau) from gate logits z (fp32), or one number per head,
+// or (state-space form) one number per head and token from a step size: dt = softplus(z_t[h] + dt_bias[h]),
+// a_t = exp(-exp(rate_log[h]) dt), the write scaled by the same step, S_t = a_t S_{t-1} + dt k_t v_t^T, and a skip term
+// skip[h] v_t added to the read-out.  q and k may have fewer heads than v (head h reads q / k head h / (heads / qk_heads)).
 //
 // One workgroup per (sequence of the step, head, block of 32 value columns): it loads the block's dk x 32 part of the
 // sequence's matrix (zero at position 0), runs the step's tokens of that sequence through it in order, and stores it
@@ -24,6 +27,8 @@ __device__ __forceinline__ float log_sigmoid_f(float z) {
   return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
 }
 
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
 template <typename QT, typename VT, int R>
 __global__ __launch_bounds__(256) void linear_recurrence_kernel(
     float* __restrict__ out, float* __restrict__ state, const QT* __restrict__ q, const QT* __restrict__ k,
@@ -31,8 +36,10 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(
     const float* __restrict__ head_decay, const int32_t* __restrict__ req_to_state, const int64_t* __restrict__ req_pool_indices,
     const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len, const int64_t* __restrict__ positions, int heads,
     int dk, int dv, int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, int64_t gate_token_stride,
-    float q_scale, float inv_tau) {
+    float q_scale, float inv_tau, int qk_heads, const float* __restrict__ dt_logits, int64_t dt_token_stride,
+    const float* __restrict__ dt_bias, const float* __restrict__ rate_log, const float* __restrict__ skip) {
   constexpr int DKP = R * RC_RG;     // key channels with padding
+  __shared__ float dts[RC_TC], das[RC_TC];
   __shared__ __attribute__((aligned(16))) float qs[RC_TC][DKP];
   __shared__ __attribute__((aligned(16))) float ks[RC_TC][DKP];
   __shared__ __attribute__((aligned(16))) float as[RC_TC][DKP];
@@ -54,17 +61,31 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(
     S[r] = (!fresh && i < dk && col < dv) ? sp[(int64_t)i * dv + col] : 0.f;
   }
   const float hd = head_decay != nullptr ? head_decay[h] : 1.f;
+  const int hq = h / (heads / qk_heads);
+  const float rate = dt_logits != nullptr ? expf(rate_log[h]) : 0.f;
+  const float skip_h = skip != nullptr ? skip[h] : 0.f;
   for (int base = 0; base < n; base += RC_TC) {
     const int m = min(RC_TC, n - base);
     __syncthreads();
+    if (dt_logits != nullptr) {
+      if (tid < m) {
+        const float dt = softplus_f(dt_logits[(t0 + base + tid) * dt_token_stride + h] + dt_bias[h]);
+        dts[tid] = dt;
+        das[tid] = expf(-rate * dt);
+      }
+      __syncthreads();
+    }
     for (int e = tid; e < m * DKP; e += 256) {
       const int tt = e / DKP, i = e - tt * DKP;
       const int64_t t = t0 + base + tt;
       float qv = 0.f, kv = 0.f, av = 1.f;
       if (i < dk) {
-        qv = to_f32(q[t * q_token_stride + (int64_t)h * dk + i]) * q_scale;
-        kv = to_f32(k[t * k_token_stride + (int64_t)h * dk + i]);
-        if (gate_logits != nullptr) {
+        qv = to_f32(q[t * q_token_stride + (int64_t)hq * dk + i]) * q_scale;
+        kv = to_f32(k[t * k_token_stride + (int64_t)hq * dk + i]);
+        if (dt_logits != nullptr) {
+          kv *= dts[tt];
+          av = das[tt];
+        } else if (gate_logits != nullptr) {
           float z = gate_logits[t * gate_token_stride + (int64_t)h * dk + i];
           if (gate_bias != nullptr) z += to_f32(gate_bias[(int64_t)h * dk + i]);
           av = expf(log_sigmoid_f(z) * inv_tau);
@@ -101,7 +122,7 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(
       acc += __shfl_xor(acc, 1, 64);
       acc += __shfl_xor(acc, 2, 64);
       acc += __shfl_xor(acc, 4, 64);
-      if (rg == 0 && col < dv) out[((t0 + base + tt) * heads + h) * (int64_t)dv + col] = acc;
+      if (rg == 0 && col < dv) out[((t0 + base + tt) * heads + h) * (int64_t)dv + col] = fmaf(skip_h, vj, acc);
     }
   }
 #pragma unroll
@@ -115,12 +136,14 @@ template <typename QT, typename VT>
 int launch_recurrence(float* out, float* state, const void* q, const void* k, const void* v, const float* gate_logits,
                       const void* gate_bias, const float* head_decay, const int32_t* req_to_state, const int64_t* req_pool_indices,
                       const int32_t* seg_start, const int32_t* seg_len, const int64_t* positions, int64_t batch, int heads, int dk,
-                      int dv, int64_t qs, int64_t ks, int64_t vs, int64_t gs, float q_scale, float tau, hipStream_t stream) {
+                      int dv, int64_t qs, int64_t ks, int64_t vs, int64_t gs, float q_scale, float tau, int qk_heads, const float* dt_logits,
+                      int64_t dts, const float* dt_bias, const float* rate_log, const float* skip, hipStream_t stream) {
   const dim3 grid((unsigned)cdiv(dv, RC_COLS), (unsigned)heads, (unsigned)batch);
 #define MI355_RC_LAUNCH(R)                                                                                                     \
   hipLaunchKernelGGL((linear_recurrence_kernel<QT, VT, R>), grid, dim3(256), 0, stream, out, state, (const QT*)q, (const QT*)k, \
                      (const VT*)v, gate_logits, (const VT*)gate_bias, head_decay, req_to_state, req_pool_indices, seg_start,   \
-                     seg_len, positions, heads, dk, dv, qs, ks, vs, gs, q_scale, 1.0f / tau)
+                     seg_len, positions, heads, dk, dv, qs, ks, vs, gs, q_scale, 1.0f / tau, qk_heads, dt_logits, dts, dt_bias,  \
+                     rate_log, skip)
   if (dk <= 32) MI355_RC_LAUNCH(4);
   else if (dk <= 64) MI355_RC_LAUNCH(8);
   else if (dk <= 128) MI355_RC_LAUNCH(16);
@@ -133,10 +156,9 @@ int launch_recurrence(float* out, float* state, const void* q, const void* k, co
 // Gated delta rule on the same layout: per token
 //     S <- diag(a_t) S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T (q_t * q_scale)
 // with a_t[i] = exp(-exp(rate_log[h]) * softplus(z_t[h, i] + rate_bias[h, i])) from fp32 logits z and beta_t = sigmoid of a
-// logit per head.  q and k may have fewer heads than v (head h reads q / k head h / (heads / qk_heads)).  A column's
+// logit per head.  With gate_per_head the decay is one number per head and token: z_t[h], rate_bias[h].  beta logits come
+// in v's type or (beta_f32) in fp32.  q and k may have fewer heads than v (head h reads q / k head h / (heads / qk_heads)).  A column's
 // S^T k and S^T q are each a sum over its eight lanes, so a token costs two rounds of lane exchanges.
-__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
-
 template <typename QT, typename VT, int R>
 __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     float* __restrict__ out, float* __restrict__ state, const QT* __restrict__ q, const QT* __restrict__ k,
@@ -144,7 +166,7 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
     const float* __restrict__ rate_bias, const float* __restrict__ rate_log, const int32_t* __restrict__ req_to_state,
     const int64_t* __restrict__ req_pool_indices, const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len,
     const int64_t* __restrict__ positions, int heads, int qk_heads, int dk, int dv, int64_t q_token_stride, int64_t k_token_stride,
-    int64_t v_token_stride, int64_t beta_token_stride, int64_t gate_token_stride, float q_scale) {
+    int64_t v_token_stride, int64_t beta_token_stride, int64_t gate_token_stride, float q_scale, int gate_per_head, int beta_f32) {
   constexpr int DKP = R * RC_RG;
   __shared__ __attribute__((aligned(16))) float qs[RC_TC][DKP];
   __shared__ __attribute__((aligned(16))) float ks[RC_TC][DKP];
@@ -179,7 +201,8 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
       if (i < dk) {
         qv = to_f32(q[t * q_token_stride + (int64_t)hq * dk + i]) * q_scale;
         kv = to_f32(k[t * k_token_stride + (int64_t)hq * dk + i]);
-        const float z = gate_logits[t * gate_token_stride + (int64_t)h * dk + i] + rate_bias[(int64_t)h * dk + i];
+        const int64_t gi = gate_per_head ? h : (int64_t)h * dk + i;
+        const float z = gate_logits[t * gate_token_stride + gi] + rate_bias[gi];
         av = expf(-rate * softplus_f(z));
       }
       qs[tt][i] = qv;
@@ -190,7 +213,11 @@ __global__ __launch_bounds__(256) void gated_delta_rule_kernel(
       const int tt = e / RC_COLS, c = e - tt * RC_COLS;
       vs[tt][c] = (c0 + c < dv) ? to_f32(v[(t0 + base + tt) * v_token_stride + (int64_t)h * dv + c0 + c]) : 0.f;
     }
-    if (tid < m) bs[tid] = 1.0f / (1.0f + expf(-to_f32(beta_logits[(t0 + base + tid) * beta_token_stride + h])));
+    if (tid < m) {
+      const int64_t bi = (t0 + base + tid) * beta_token_stride + h;
+      const float bl = beta_f32 ? reinterpret_cast<const float*>(beta_logits)[bi] : to_f32(beta_logits[bi]);
+      bs[tid] = 1.0f / (1.0f + expf(-bl));
+    }
     __syncthreads();
     for (int tt = 0; tt < m; ++tt) {
       float dot = 0.f;
@@ -243,12 +270,12 @@ int launch_delta(float* out, float* state, const void* q, const void* k, const v
                  const float* gate_logits, const float* rate_bias, const float* rate_log, const int32_t* req_to_state,
                  const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len, const int64_t* positions,
                  int64_t batch, int heads, int qk_heads, int dk, int dv, int64_t qs, int64_t ks, int64_t vs, int64_t bs, int64_t gs,
-                 float q_scale, hipStream_t stream) {
+                 float q_scale, int gate_per_head, int beta_f32, hipStream_t stream) {
   const dim3 grid((unsigned)cdiv(dv, RC_COLS), (unsigned)heads, (unsigned)batch);
 #define MI355_GD_LAUNCH(R)                                                                                                     \
   hipLaunchKernelGGL((gated_delta_rule_kernel<QT, VT, R>), grid, dim3(256), 0, stream, out, state, (const QT*)q, (const QT*)k,  \
                      (const VT*)v, (const VT*)beta_logits, gate_logits, rate_bias, rate_log, req_to_state, req_pool_indices,   \
-                     seg_start, seg_len, positions, heads, qk_heads, dk, dv, qs, ks, vs, bs, gs, q_scale)
+                     seg_start, seg_len, positions, heads, qk_heads, dk, dv, qs, ks, vs, bs, gs, q_scale, gate_per_head, beta_f32)
   if (dk <= 32) MI355_GD_LAUNCH(4);
   else if (dk <= 64) MI355_GD_LAUNCH(8);
   else if (dk <= 128) MI355_GD_LAUNCH(16);
@@ -268,14 +295,31 @@ int mi355_linear_recurrence(float* out, float* state, const void* q, const void*
                             const int64_t* positions, int64_t batch, int heads, int key_dim, int value_dim, int64_t q_token_stride,
                             int64_t k_token_stride, int64_t v_token_stride, int64_t gate_token_stride, float q_scale, float tau,
                             int qk_dtype, int v_dtype, void* stream) {
-  MI355_REQUIRE(out && state && q && k && v && req_to_state && req_pool_indices && positions, MI355_ERR_INVALID,
-                "linear_recurrence: null pointer");
   MI355_REQUIRE((gate_logits != nullptr) != (head_decay != nullptr), MI355_ERR_INVALID,
                 "linear_recurrence: the decay is either gate logits per channel or one number per head");
+  return mi355_linear_recurrence_ssm(out, state, q, k, v, gate_logits, gate_bias, head_decay, nullptr, 0, nullptr, nullptr, nullptr,
+                                     req_to_state, req_pool_indices, seg_start, seg_len, positions, batch, heads, heads, key_dim,
+                                     value_dim, q_token_stride, k_token_stride, v_token_stride, gate_token_stride, q_scale, tau,
+                                     qk_dtype, v_dtype, stream);
+}
+
+int mi355_linear_recurrence_ssm(float* out, float* state, const void* q, const void* k, const void* v, const float* gate_logits,
+                                const void* gate_bias, const float* head_decay, const float* dt_logits, int64_t dt_token_stride,
+                                const float* dt_bias, const float* rate_log, const float* skip, const int32_t* req_to_state,
+                                const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                                const int64_t* positions, int64_t batch, int heads, int qk_heads, int key_dim, int value_dim,
+                                int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, int64_t gate_token_stride,
+                                float q_scale, float tau, int qk_dtype, int v_dtype, void* stream) {
+  MI355_REQUIRE(out && state && q && k && v && req_to_state && req_pool_indices && positions, MI355_ERR_INVALID,
+                "linear_recurrence: null pointer");
+  MI355_REQUIRE((gate_logits != nullptr) + (head_decay != nullptr) + (dt_logits != nullptr) == 1, MI355_ERR_INVALID,
+                "linear_recurrence: the decay is gate logits per channel, one number per head, or a step size per head and token");
+  MI355_REQUIRE(dt_logits == nullptr || (dt_bias && rate_log && dt_token_stride >= heads), MI355_ERR_INVALID,
+                "linear_recurrence: step sizes come with their bias and the heads' rates");
   MI355_REQUIRE((seg_start == nullptr) == (seg_len == nullptr), MI355_ERR_INVALID,
                 "linear_recurrence: seg_start and seg_len come together");
-  MI355_REQUIRE(batch >= 0 && batch <= 65535 && heads > 0 && heads <= 65535 && key_dim > 0 && value_dim > 0 && tau > 0.f,
-                MI355_ERR_INVALID, "linear_recurrence: bad shape");
+  MI355_REQUIRE(batch >= 0 && batch <= 65535 && heads > 0 && heads <= 65535 && key_dim > 0 && value_dim > 0 && tau > 0.f &&
+                    qk_heads > 0 && heads % qk_heads == 0, MI355_ERR_INVALID, "linear_recurrence: bad shape");
   MI355_REQUIRE(key_dim <= 256, MI355_ERR_UNSUPPORTED, "linear_recurrence: key width %d above 256", key_dim);
   MI355_REQUIRE(qk_dtype == v_dtype || qk_dtype == MI355_F32, MI355_ERR_UNSUPPORTED,
                 "linear_recurrence: q and k come in the type of v or in fp32");
@@ -285,11 +329,13 @@ int mi355_linear_recurrence(float* out, float* state, const void* q, const void*
     if (qk_dtype == v_dtype)
       rc = launch_recurrence<T, T>(out, state, q, k, v, gate_logits, gate_bias, head_decay, req_to_state, req_pool_indices,
                                    seg_start, seg_len, positions, batch, heads, key_dim, value_dim, q_token_stride, k_token_stride,
-                                   v_token_stride, gate_token_stride, q_scale, tau, (hipStream_t)stream);
+                                   v_token_stride, gate_token_stride, q_scale, tau, qk_heads, dt_logits, dt_token_stride, dt_bias,
+                                   rate_log, skip, (hipStream_t)stream);
     else
       rc = launch_recurrence<float, T>(out, state, q, k, v, gate_logits, gate_bias, head_decay, req_to_state, req_pool_indices,
                                        seg_start, seg_len, positions, batch, heads, key_dim, value_dim, q_token_stride,
-                                       k_token_stride, v_token_stride, gate_token_stride, q_scale, tau, (hipStream_t)stream);
+                                       k_token_stride, v_token_stride, gate_token_stride, q_scale, tau, qk_heads, dt_logits,
+                                       dt_token_stride, dt_bias, rate_log, skip, (hipStream_t)stream);
   });
   if (rc != MI355_OK) return rc;
   MI355_CHECK_LAUNCH("linear_recurrence");
@@ -302,6 +348,19 @@ int mi355_gated_delta_rule(float* out, float* state, const void* q, const void* 
                            const int64_t* positions, int64_t batch, int heads, int qk_heads, int key_dim, int value_dim,
                            int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, int64_t beta_token_stride,
                            int64_t gate_token_stride, float q_scale, int qk_dtype, int v_dtype, void* stream) {
+  return mi355_gated_delta_rule_ex(out, state, q, k, v, beta_logits, gate_logits, rate_bias, rate_log, req_to_state, req_pool_indices,
+                                   seg_start, seg_len, positions, batch, heads, qk_heads, key_dim, value_dim, q_token_stride,
+                                   k_token_stride, v_token_stride, beta_token_stride, gate_token_stride, q_scale, 0, 0, qk_dtype,
+                                   v_dtype, stream);
+}
+
+int mi355_gated_delta_rule_ex(float* out, float* state, const void* q, const void* k, const void* v, const void* beta_logits,
+                              const float* gate_logits, const float* rate_bias, const float* rate_log, const int32_t* req_to_state,
+                              const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                              const int64_t* positions, int64_t batch, int heads, int qk_heads, int key_dim, int value_dim,
+                              int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, int64_t beta_token_stride,
+                              int64_t gate_token_stride, float q_scale, int gate_per_head, int beta_f32, int qk_dtype, int v_dtype,
+                              void* stream) {
   MI355_REQUIRE(out && state && q && k && v && beta_logits && gate_logits && rate_bias && rate_log && req_to_state &&
                     req_pool_indices && positions, MI355_ERR_INVALID, "gated_delta_rule: null pointer");
   MI355_REQUIRE((seg_start == nullptr) == (seg_len == nullptr), MI355_ERR_INVALID,
@@ -317,12 +376,13 @@ int mi355_gated_delta_rule(float* out, float* state, const void* q, const void* 
     if (qk_dtype == v_dtype)
       rc = launch_delta<T, T>(out, state, q, k, v, beta_logits, gate_logits, rate_bias, rate_log, req_to_state, req_pool_indices,
                               seg_start, seg_len, positions, batch, heads, qk_heads, key_dim, value_dim, q_token_stride,
-                              k_token_stride, v_token_stride, beta_token_stride, gate_token_stride, q_scale, (hipStream_t)stream);
+                              k_token_stride, v_token_stride, beta_token_stride, gate_token_stride, q_scale, gate_per_head, beta_f32,
+                              (hipStream_t)stream);
     else
       rc = launch_delta<float, T>(out, state, q, k, v, beta_logits, gate_logits, rate_bias, rate_log, req_to_state,
                                   req_pool_indices, seg_start, seg_len, positions, batch, heads, qk_heads, key_dim, value_dim,
                                   q_token_stride, k_token_stride, v_token_stride, beta_token_stride, gate_token_stride, q_scale,
-                                  (hipStream_t)stream);
+                                  gate_per_head, beta_f32, (hipStream_t)stream);
   });
   if (rc != MI355_OK) return rc;
   MI355_CHECK_LAUNCH("gated_delta_rule");

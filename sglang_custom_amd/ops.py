@@ -1283,23 +1283,41 @@ def scaled_add_group_rmsnorm(x: torch.Tensor, branch: Optional[torch.Tensor], al
     return x if h is None else h
 
 
-def rmsnorm_residual_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
-    """x += y / sqrt(mean(y^2) + eps) * weight in place on the fp32 rows; returns the new x in the weight's dtype."""
-    _gpu(x, y, weight)
+def rmsnorm_residual_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, offset: float = 0.0,
+                         layer_scale: Optional[torch.Tensor] = None, mult: float = 1.0) -> torch.Tensor:
+    """x += mult * layer_scale * y / sqrt(mean(y^2) + eps) * (offset + weight) in place on the fp32 rows (layer_scale [D] or
+    None); returns the new x in the weight's dtype."""
+    _gpu(x, y, weight, layer_scale)
     assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and y.shape == x.shape and y.stride(1) == 1
     assert y.dtype == weight.dtype and weight.is_contiguous() and weight.numel() == x.shape[1]
+    assert layer_scale is None or (layer_scale.dtype == weight.dtype and layer_scale.is_contiguous() and layer_scale.numel() == x.shape[1])
     T, D = x.shape
     h = None if weight.dtype == torch.float32 else torch.empty((T, D), dtype=weight.dtype, device=x.device)
-    check(_lib_().mi355_rmsnorm_residual_add(x.data_ptr(), _p(h), y.data_ptr(), y.stride(0), weight.data_ptr(), T, D, float(eps),
-                                             _dt(weight), _stream(x)), "rmsnorm_residual_add")
+    check(_lib_().mi355_rmsnorm_residual_add_scaled(x.data_ptr(), _p(h), y.data_ptr(), y.stride(0), weight.data_ptr(), _p(layer_scale),
+                                                    float(offset), float(mult), T, D, float(eps), _dt(weight), _stream(x)),
+          "rmsnorm_residual_add")
     return x if h is None else h
+
+
+def gated_group_rmsnorm(y: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, groups: int, eps: float) -> torch.Tensor:
+    """fp32 rows y [T, D], gate [T, D] (row-strided, the weight's dtype) -> N(y * silu(gate)) * weight with N the RMS norm over
+    `groups` equal consecutive parts of the row: gated first, normed after.  Result in the weight's dtype."""
+    _gpu(y, gate, weight)
+    T, D = y.shape
+    assert y.dtype == torch.float32 and y.is_contiguous() and gate.shape == (T, D) and gate.stride(1) == 1
+    assert gate.dtype == weight.dtype and weight.is_contiguous() and weight.numel() == D and D % groups == 0
+    out = torch.empty((T, D), dtype=weight.dtype, device=y.device)
+    check(_lib_().mi355_gated_group_rmsnorm(out.data_ptr(), y.data_ptr(), gate.data_ptr(), gate.stride(0), weight.data_ptr(), T, D,
+                                            int(groups), float(eps), _dt(weight), _stream(y)), "gated_group_rmsnorm")
+    return out
 
 
 def head_norm_rope(src: torch.Tensor, weight: Optional[torch.Tensor], eps: float, positions: torch.Tensor, inv_freq: torch.Tensor,
                    rot_dims: int, interleaved: bool, scale: float, out_dtype: torch.dtype, cache: Optional[torch.Tensor] = None,
-                   loc: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """src [T, H, d] (token / head strides free) -> optional RMS norm per head, rotation of the first rot_dims features,
-    scale; to a new [T, H, d] tensor of out_dtype, or into cache[loc[t]] ([slots, H, d]) when a cache is given."""
+                   loc: Optional[torch.Tensor] = None, rot_mag: float = 1.0) -> torch.Tensor:
+    """src [T, H, d] (token / head strides free) -> optional RMS norm per head, rotation of the first rot_dims features (cos
+    and sin times rot_mag), scale; to a new [T, H, d] tensor of out_dtype, or into cache[loc[t]] ([slots, H, d]) when a cache
+    is given."""
     _gpu(src, weight, positions, inv_freq, cache, loc)
     T, H, d = src.shape
     assert src.stride(2) == 1 and positions.dtype == torch.int64 and positions.is_contiguous()
@@ -1312,10 +1330,34 @@ def head_norm_rope(src: torch.Tensor, weight: Optional[torch.Tensor], eps: float
     else:
         out = torch.empty((T, H, d), dtype=out_dtype, device=src.device)
         loc = None
-    check(_lib_().mi355_head_norm_rope(out.data_ptr(), src.data_ptr(), _p(weight), positions.data_ptr(), _p(loc),
-                                       _p(inv_freq) if rot_dims else None, T, H, d, src.stride(0), src.stride(1), out.stride(0),
-                                       out.stride(1), out.shape[0], int(rot_dims), int(bool(interleaved)), float(scale),
-                                       float(eps), _dt(src), _DT[out_dtype], _stream(src)), "head_norm_rope")
+    check(_lib_().mi355_head_norm_rope_mag(out.data_ptr(), src.data_ptr(), _p(weight), positions.data_ptr(), _p(loc),
+                                           _p(inv_freq) if rot_dims else None, T, H, d, src.stride(0), src.stride(1), out.stride(0),
+                                           out.stride(1), out.shape[0], int(rot_dims), int(bool(interleaved)), float(scale),
+                                           float(eps), float(rot_mag), _dt(src), _DT[out_dtype], _stream(src)), "head_norm_rope")
+    return out
+
+
+def qkv_norm_rope_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, eps: float,
+                        positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot_dims: int, interleaved: bool, rot_mag: float,
+                        k_cache: torch.Tensor, v_cache: torch.Tensor, loc: torch.Tensor) -> torch.Tensor:
+    """The three head norms of an attention layer in one launch: q [T, H, d], k [T, G, d], v [T, G, dv] (column blocks of one
+    projection's output will do).  Returns head_norm_rope(q, wq, ...) as a new [T, H, d]; head_norm_rope(k, wk, ...) goes into
+    k_cache[loc], v / rms(v) into v_cache[loc]."""
+    _gpu(q, k, v, wq, wk, positions, inv_freq, k_cache, v_cache, loc)
+    T, H, d = q.shape
+    G, dv = k.shape[1], v.shape[2]
+    assert k.shape == (T, G, d) and v.shape == (T, G, dv) and q.dtype == k.dtype == v.dtype == k_cache.dtype == v_cache.dtype
+    for t_ in (q, k, v):
+        assert t_.stride(2) == 1 and t_.stride(1) == t_.shape[2], "heads lie side by side in a token's row"
+    assert wq.dtype == q.dtype and wk.dtype == q.dtype and wq.numel() == d and wk.numel() == d and wq.is_contiguous() and wk.is_contiguous()
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape[1:] == (G, d) and v_cache.shape[1:] == (G, dv)
+    assert positions.dtype == torch.int64 and positions.is_contiguous() and loc.dtype == torch.int64 and loc.is_contiguous() and loc.numel() == T
+    assert rot_dims == 0 or (inv_freq.dtype == torch.float32 and inv_freq.numel() >= rot_dims // 2)
+    out = torch.empty((T, H, d), dtype=q.dtype, device=q.device)
+    check(_lib_().mi355_qkv_norm_rope_write(out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                            q.stride(0), k.stride(0), v.stride(0), wq.data_ptr(), wk.data_ptr(), positions.data_ptr(),
+                                            loc.data_ptr(), _p(inv_freq) if rot_dims else None, T, H, G, d, dv, int(rot_dims),
+                                            int(bool(interleaved)), float(eps), float(rot_mag), _dt(q), _stream(q)), "qkv_norm_rope_write")
     return out
 
 
@@ -1348,21 +1390,31 @@ def gelu_tanh_mul_rows(gate: torch.Tensor, table: torch.Tensor, ids: torch.Tenso
 def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
                       req_to_state: torch.Tensor, req_pool_indices: torch.Tensor, positions: torch.Tensor, q_scale: float,
                       gate_logits: Optional[torch.Tensor] = None, gate_bias: Optional[torch.Tensor] = None, tau: float = 1.0,
-                      head_decay: Optional[torch.Tensor] = None, tok_req=None, seg_start=None, seg_len=None) -> torch.Tensor:
+                      head_decay: Optional[torch.Tensor] = None, tok_req=None, seg_start=None, seg_len=None,
+                      dt_logits: Optional[torch.Tensor] = None, dt_bias: Optional[torch.Tensor] = None,
+                      rate_log: Optional[torch.Tensor] = None, skip: Optional[torch.Tensor] = None) -> torch.Tensor:
     """S = diag(a) S + k v^T, out = S^T (q * q_scale) per head over every sequence's tokens of the step, on
     state[slot] ([slots, H, dk, dv] fp32, read unless the sequence starts at position 0, written back).  q, k [T, H, dk]
-    (fp32 or v's dtype), v [T, H, dv]; the decay from gate_logits fp32 [T, H * dk] (+ gate_bias, / tau) or head_decay fp32 [H]."""
-    _gpu(q, k, v, out, state, req_to_state, req_pool_indices, positions, gate_logits, gate_bias, head_decay)
-    T, H, dk = q.shape
-    dv = v.shape[2]
-    assert k.shape == q.shape and v.shape[:2] == (T, H) and q.dtype == k.dtype and q.dtype in (v.dtype, torch.float32)
+    (fp32 or v's dtype), v [T, H, dv]; the decay from gate_logits fp32 [T, H * dk] (+ gate_bias, / tau) or head_decay fp32 [H],
+    or (state-space form) from step sizes: dt = softplus(dt_logits [T, H] + dt_bias [H]), a = exp(-exp(rate_log [H]) dt),
+    S = a S + dt k v^T, out += skip [H] * v (all fp32).  q and k may have G < H heads (head h reads head h // (H / G))."""
+    _gpu(q, k, v, out, state, req_to_state, req_pool_indices, positions, gate_logits, gate_bias, head_decay, dt_logits, dt_bias,
+         rate_log, skip)
+    T, G, dk = q.shape
+    H, dv = v.shape[1], v.shape[2]
+    assert k.shape == q.shape and v.shape[0] == T and H % G == 0 and q.dtype == k.dtype and q.dtype in (v.dtype, torch.float32)
     for t in (q, k, v):
         assert t.stride(2) == 1 and t.stride(1) == t.shape[2], "heads lie side by side in a token's row"
     assert out.dtype == torch.float32 and out.shape == (T, H, dv) and out.is_contiguous()
     assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dk, dv)
     assert req_to_state.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
-    assert (gate_logits is None) != (head_decay is None)
-    if gate_logits is not None:
+    assert (gate_logits is not None) + (head_decay is not None) + (dt_logits is not None) == 1
+    if dt_logits is not None:
+        assert dt_logits.dtype == torch.float32 and dt_logits.shape == (T, H) and dt_logits.stride(1) == 1
+        for w in (dt_bias, rate_log, skip):
+            assert w is None or (w.dtype == torch.float32 and w.numel() == H and w.is_contiguous())
+        assert dt_bias is not None and rate_log is not None
+    elif gate_logits is not None:
         assert gate_logits.dtype == torch.float32 and gate_logits.shape == (T, H * dk) and gate_logits.stride(1) == 1
         assert gate_bias is None or (gate_bias.dtype == v.dtype and gate_bias.numel() == H * dk and gate_bias.is_contiguous())
     else:
@@ -1370,11 +1422,13 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: to
     _, ss, sl = _seg(tok_req, seg_start, seg_len)
     B = req_pool_indices.numel()
     assert seg_start is not None or B == T, "without segments every token is a sequence of its own"
-    check(_lib_().mi355_linear_recurrence(out.data_ptr(), state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                          _p(gate_logits), _p(gate_bias), _p(head_decay), req_to_state.data_ptr(),
-                                          req_pool_indices.data_ptr(), ss, sl, positions.data_ptr(), B, H, dk, dv, q.stride(0),
-                                          k.stride(0), v.stride(0), gate_logits.stride(0) if gate_logits is not None else 0,
-                                          float(q_scale), float(tau), _dt(q), _dt(v), _stream(q)), "linear_recurrence")
+    check(_lib_().mi355_linear_recurrence_ssm(out.data_ptr(), state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                              _p(gate_logits), _p(gate_bias), _p(head_decay), _p(dt_logits),
+                                              dt_logits.stride(0) if dt_logits is not None else 0, _p(dt_bias), _p(rate_log), _p(skip),
+                                              req_to_state.data_ptr(), req_pool_indices.data_ptr(), ss, sl, positions.data_ptr(), B,
+                                              H, G, dk, dv, q.stride(0), k.stride(0), v.stride(0),
+                                              gate_logits.stride(0) if gate_logits is not None else 0, float(q_scale), float(tau),
+                                              _dt(q), _dt(v), _stream(q)), "linear_recurrence")
     return out
 
 
@@ -1553,14 +1607,15 @@ ACTIVATIONS = {"none": 0, "silu": 1, "relu2": 2}
 
 def causal_conv(u: torch.Tensor, w1: torch.Tensor, state: torch.Tensor, req_to_state: torch.Tensor, req_pool_indices: torch.Tensor,
                 positions: torch.Tensor, w2: Optional[torch.Tensor] = None, residual: bool = False, act: str = "none",
-                tok_req=None, seg_start=None, seg_len=None):
+                tok_req=None, seg_start=None, seg_len=None, bias: Optional[torch.Tensor] = None):
     """Causal convolution over time per channel of u [T, C] (row-strided) with filter w1 [C, taps] (last column: the current
     token) and, optionally, a second filter w2 over the same input; with `residual`, u is added to each result; then `act`.
     Inputs before a step's first token of a sequence come from state[slot] (fp32 [slots, taps - 1, C]; zeros before position
     0); afterwards the state holds the sequence's last taps - 1 inputs.  Returns y1, or (y1, y2)."""
-    _gpu(u, w1, w2, state, req_to_state, req_pool_indices, positions)
+    _gpu(u, w1, w2, state, req_to_state, req_pool_indices, positions, bias)
     T, C = u.shape
     taps = w1.shape[1]
+    assert bias is None or (bias.dtype == u.dtype and bias.numel() == C and bias.is_contiguous()), "bias [C] of the first filter"
     assert u.stride(1) == 1 and w1.shape == (C, taps) and w1.is_contiguous() and w1.dtype == u.dtype
     assert w2 is None or (w2.shape == w1.shape and w2.is_contiguous() and w2.dtype == u.dtype)
     assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (taps - 1, C)
@@ -1571,9 +1626,10 @@ def causal_conv(u: torch.Tensor, w1: torch.Tensor, state: torch.Tensor, req_to_s
     tr, ss, sl = _seg(tok_req, seg_start, seg_len)
     assert seg_start is not None or req_pool_indices.numel() == T, "without segments every token is a sequence of its own"
     lib = _lib_()
-    check(lib.mi355_causal_conv(y1.data_ptr(), _p(y2), u.data_ptr(), u.stride(0), w1.data_ptr(), _p(w2), _p(state) if taps > 1 else None,
-                                req_to_state.data_ptr(), req_pool_indices.data_ptr(), tr, ss, positions.data_ptr(), T, C, taps,
-                                int(bool(residual)), ACTIVATIONS[act], _dt(u), _stream(u)), "causal_conv")
+    check(lib.mi355_causal_conv_bias(y1.data_ptr(), _p(y2), u.data_ptr(), u.stride(0), w1.data_ptr(), _p(w2), _p(bias),
+                                     _p(state) if taps > 1 else None, req_to_state.data_ptr(), req_pool_indices.data_ptr(), tr, ss,
+                                     positions.data_ptr(), T, C, taps, int(bool(residual)), ACTIVATIONS[act], _dt(u), _stream(u)),
+          "causal_conv")
     if seg_start is not None and taps > 1:
         check(lib.mi355_causal_conv_state_update(state.data_ptr(), u.data_ptr(), u.stride(0), req_to_state.data_ptr(),
                                                  req_pool_indices.data_ptr(), ss, sl, positions.data_ptr(), req_pool_indices.numel(),
@@ -1597,17 +1653,19 @@ def gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_log
                      tok_req=None, seg_start=None, seg_len=None) -> torch.Tensor:
     """Per head  S = diag(a) S;  u = beta (v - S^T k);  S += k u^T;  out = S^T (q * q_scale)  over every sequence's tokens of the
     step on state[slot] ([slots, H, dk, dv] fp32).  q, k [T, G, dk] (fp32 or v's dtype; head h reads head h // (H / G)), v
-    [T, H, dv], beta_logits [T, H] (row-strided, v's dtype), gate_logits fp32 [T, H * dk], rate_bias fp32 [H * dk], rate_log
-    fp32 [H]:  a = exp(-exp(rate_log) * softplus(gate_logits + rate_bias)),  beta = sigmoid(beta_logits)."""
+    [T, H, dv], beta_logits [T, H] (row-strided, v's dtype or fp32), gate_logits fp32 [T, H * dk], rate_bias fp32 [H * dk],
+    rate_log fp32 [H]:  a = exp(-exp(rate_log) * softplus(gate_logits + rate_bias)),  beta = sigmoid(beta_logits).  With
+    gate_logits [T, H] and rate_bias [H] the decay is one number per head and token."""
     _gpu(q, k, v, beta_logits, gate_logits, rate_bias, rate_log, out, state, req_to_state, req_pool_indices, positions)
     T, G, dk = q.shape
     H, dv = v.shape[1], v.shape[2]
     assert k.shape == q.shape and v.shape[0] == T and H % G == 0 and q.dtype == k.dtype and q.dtype in (v.dtype, torch.float32)
     for t in (q, k, v):
         assert t.stride(2) == 1 and t.stride(1) == t.shape[2], "heads lie side by side in a token's row"
-    assert beta_logits.shape == (T, H) and beta_logits.stride(1) == 1 and beta_logits.dtype == v.dtype
-    assert gate_logits.dtype == torch.float32 and gate_logits.shape == (T, H * dk) and gate_logits.stride(1) == 1
-    assert rate_bias.dtype == torch.float32 and rate_bias.numel() == H * dk and rate_bias.is_contiguous()
+    assert beta_logits.shape == (T, H) and beta_logits.stride(1) == 1 and beta_logits.dtype in (v.dtype, torch.float32)
+    per_head = gate_logits.shape[1] == H and rate_bias.numel() == H
+    assert gate_logits.dtype == torch.float32 and gate_logits.shape == (T, H if per_head else H * dk) and gate_logits.stride(1) == 1
+    assert rate_bias.dtype == torch.float32 and rate_bias.numel() == (H if per_head else H * dk) and rate_bias.is_contiguous()
     assert rate_log.dtype == torch.float32 and rate_log.numel() == H and rate_log.is_contiguous()
     assert out.dtype == torch.float32 and out.shape == (T, H, dv) and out.is_contiguous()
     assert state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, dk, dv)
@@ -1615,11 +1673,12 @@ def gated_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta_log
     _, ss, sl = _seg(tok_req, seg_start, seg_len)
     B = req_pool_indices.numel()
     assert seg_start is not None or B == T, "without segments every token is a sequence of its own"
-    check(_lib_().mi355_gated_delta_rule(out.data_ptr(), state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                         beta_logits.data_ptr(), gate_logits.data_ptr(), rate_bias.data_ptr(), rate_log.data_ptr(),
-                                         req_to_state.data_ptr(), req_pool_indices.data_ptr(), ss, sl, positions.data_ptr(), B, H, G,
-                                         dk, dv, q.stride(0), k.stride(0), v.stride(0), beta_logits.stride(0), gate_logits.stride(0),
-                                         float(q_scale), _dt(q), _dt(v), _stream(q)), "gated_delta_rule")
+    check(_lib_().mi355_gated_delta_rule_ex(out.data_ptr(), state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                            beta_logits.data_ptr(), gate_logits.data_ptr(), rate_bias.data_ptr(), rate_log.data_ptr(),
+                                            req_to_state.data_ptr(), req_pool_indices.data_ptr(), ss, sl, positions.data_ptr(), B, H, G,
+                                            dk, dv, q.stride(0), k.stride(0), v.stride(0), beta_logits.stride(0), gate_logits.stride(0),
+                                            float(q_scale), int(per_head), int(beta_logits.dtype == torch.float32 and v.dtype != torch.float32),
+                                            _dt(q), _dt(v), _stream(q)), "gated_delta_rule")
     return out
 
 
@@ -1628,23 +1687,35 @@ def window_attention_block_tokens(heads: int, kv_heads: int, head_dim: int, v_he
     return int(_lib_().mi355_window_attention_block_tokens(heads, kv_heads, head_dim, v_head_dim, _DT[dtype]))
 
 
-def window_attention_splits(tokens: int, heads: int, kv_heads: int, max_len: int, window: int, dtype: torch.dtype) -> int:
+def window_attention_splits(tokens: int, heads: int, kv_heads: int, max_len: int, window: int, dtype: torch.dtype, pool: int = 0) -> int:
     """Key ranges per token for a decode-sized launch: two workgroups per CU, at least 256 visible keys each.  Measured on
     MI355X (64 sequences x 1024 keys, heads of 128): with 256 workgroups two ranges take 0.64 of one range's time, four 0.76,
     eight as long as one; with 512 workgroups one range is best -- every further range adds a workgroup's fixed cost (its
     query tile, its partial results and their merge) to a walk that is short already."""
     wgs = max(1, tokens * kv_heads * ((heads // kv_heads + 63) // 64))
     seen = min(max_len, window) if window > 0 else max_len
+    if pool > 0 and window > 0:
+        seen += max(0, max_len - window) // pool        # the averaged blocks before the window
     return int(max(1, min(64, 512 // wgs, seen // 256)))
 
 
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, req_to_token: torch.Tensor,
                      req_pool_indices: torch.Tensor, positions: torch.Tensor, sink: Optional[torch.Tensor], window: int, scale: float,
-                     tok_req=None, blocks=None, max_run: Optional[int] = None, num_splits: int = 1) -> torch.Tensor:
+                     tok_req=None, blocks=None, max_run: Optional[int] = None, num_splits: int = 1, pool: int = 0,
+                     pooled_k: Optional[torch.Tensor] = None, pooled_v: Optional[torch.Tensor] = None, pool_div: int = 1,
+                     head_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention of q [T, H, d] over the keys within `window` positions (0: all earlier ones) in caches
     [slots, G, d] / [slots, G, dv], with exp(sink[h]) added to the denominator (sink fp32 [H] or None) -> out [T, H, dv];
-    blocks int32 [n, 2] runs of at most max_run consecutive tokens of one sequence, or None (one token per run)."""
-    _gpu(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, sink, tok_req, blocks)
+    blocks int32 [n, 2] runs of at most max_run consecutive tokens of one sequence, or None (one token per run).
+    pool > 0: a token at position i also sees the averaged row of every block b of `pool` positions with
+    b pool + pool - 1 <= i - window, at pooled_k / pooled_v [slot(b pool + pool - 1) // pool_div].  head_gate [T, H]
+    (row-strided logits): head h's result times their sigmoid."""
+    _gpu(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, sink, tok_req, blocks, pooled_k, pooled_v, head_gate)
+    if pool > 0:
+        assert window > 0 and pooled_k is not None and pooled_v is not None and pool_div in (1, pool)
+        assert pooled_k.is_contiguous() and pooled_v.is_contiguous() and pooled_k.dtype == pooled_v.dtype == k_cache.dtype
+        assert pooled_k.shape[1:] == k_cache.shape[1:] and pooled_v.shape[1:] == v_cache.shape[1:]
+    assert head_gate is None or (head_gate.shape == q.shape[:2] and head_gate.stride(1) == 1 and head_gate.dtype == q.dtype)
     T, H, d = q.shape
     G, dv = k_cache.shape[1], v_cache.shape[2]
     assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape[2] == d and v_cache.shape[1] == G
@@ -1659,12 +1730,33 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     else:
         nb, max_run = T, 1
     scratch = torch.empty(num_splits * T * H * (dv + 2), dtype=torch.float32, device=q.device) if num_splits > 1 else None
-    check(_lib_().mi355_window_attention(
-        out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), req_to_token.data_ptr(), req_pool_indices.data_ptr(),
-        _p(tok_req), positions.data_ptr(), _p(blocks), nb, _p(sink), q.stride(0), q.stride(1), out.stride(0), out.stride(1),
-        req_to_token.stride(0), H, G, d, dv, int(window), float(scale), int(num_splits), _p(scratch), T, int(max_run), _dt(q), _stream(q)),
-          "window_attention")
+    check(_lib_().mi355_window_attention_pooled(
+        out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _p(pooled_k) if pool > 0 else None,
+        _p(pooled_v) if pool > 0 else None, req_to_token.data_ptr(), req_pool_indices.data_ptr(), _p(tok_req), positions.data_ptr(),
+        _p(blocks), nb, _p(sink), _p(head_gate), head_gate.stride(0) if head_gate is not None else 0, q.stride(0), q.stride(1),
+        out.stride(0), out.stride(1), req_to_token.stride(0), H, G, d, dv, int(window), int(pool), int(pool_div), float(scale),
+        int(num_splits), _p(scratch), T, int(max_run), _dt(q), _stream(q)), "window_attention")
     return out
+
+
+def pool_kv_blocks(k_cache: torch.Tensor, v_cache: torch.Tensor, pooled_k: torch.Tensor, pooled_v: torch.Tensor,
+                   req_to_token: torch.Tensor, req_pool_indices: torch.Tensor, positions: torch.Tensor, pool: int, pool_div: int = 1,
+                   tok_req=None) -> None:
+    """For every token of the step whose position p ends a block of `pool` positions ((p + 1) % pool == 0): the mean of the
+    block's cached keys (values) goes to pooled_k (pooled_v) [slot(p) // pool_div].  The step's keys and values must be in
+    the caches already."""
+    _gpu(k_cache, v_cache, pooled_k, pooled_v, req_to_token, req_pool_indices, positions, tok_req)
+    G, d, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and pooled_k.is_contiguous() and pooled_v.is_contiguous()
+    assert pooled_k.shape[1:] == (G, d) and pooled_v.shape[1:] == (G, dv) and pooled_k.dtype == pooled_v.dtype == k_cache.dtype == v_cache.dtype
+    assert req_to_token.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
+    assert pool >= 1 and pool_div in (1, pool) and pooled_k.shape[0] * pool_div >= k_cache.shape[0]
+    T = positions.numel()
+    assert tok_req is None or (tok_req.dtype == torch.int32 and tok_req.numel() == T)
+    check(_lib_().mi355_pool_kv_blocks(pooled_k.data_ptr(), pooled_v.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                       req_to_token.data_ptr(), req_pool_indices.data_ptr(), _p(tok_req), positions.data_ptr(), T,
+                                       req_to_token.stride(0), G, d, dv, int(pool), int(pool_div), _dt(k_cache), _stream(k_cache)),
+          "pool_kv_blocks")
 
 
 def moe_route_scores(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, n_groups: int, keep_groups: int, scale: float,

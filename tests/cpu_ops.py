@@ -349,13 +349,24 @@ def scaled_add_group_rmsnorm(x, branch, alpha, weight, groups, eps, rows=None, c
     return n.to(weight.dtype)
 
 
-def rmsnorm_residual_add(x, y, weight, eps):
+def rmsnorm_residual_add(x, y, weight, eps, offset=0.0, layer_scale=None, mult=1.0):
     y = y.float()
-    x.add_(y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps) * weight.float())
+    n = y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps) * (offset + weight.float())
+    if layer_scale is not None:
+        n = n * layer_scale.float()
+    x.add_(mult * n)
     return x if weight.dtype == torch.float32 else x.to(weight.dtype)
 
 
-def head_norm_rope(src, weight, eps, positions, inv_freq, rot_dims, interleaved, scale, out_dtype, cache=None, loc=None):
+def gated_group_rmsnorm(y, gate, weight, groups, eps):
+    T, D = y.shape
+    g = gate.float()
+    v = (y * (g * torch.sigmoid(g))).view(T, groups, D // groups)
+    n = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)
+    return (n.reshape(T, D) * weight.float()).to(weight.dtype)
+
+
+def head_norm_rope(src, weight, eps, positions, inv_freq, rot_dims, interleaved, scale, out_dtype, cache=None, loc=None, rot_mag=1.0):
     T, H, d = src.shape
     out = torch.empty((T, H, d), dtype=torch.float32)
     for t in range(T):
@@ -364,7 +375,7 @@ def head_norm_rope(src, weight, eps, positions, inv_freq, rot_dims, interleaved,
             v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight.float()
         if rot_dims:
             ang = float(positions[t]) * inv_freq[: rot_dims // 2].float()
-            c, s = torch.cos(ang), torch.sin(ang)
+            c, s = torch.cos(ang) * rot_mag, torch.sin(ang) * rot_mag
             r = v.clone()
             if interleaved:
                 a, b = v[:, 0:rot_dims:2], v[:, 1:rot_dims:2]
@@ -380,21 +391,37 @@ def head_norm_rope(src, weight, eps, positions, inv_freq, rot_dims, interleaved,
     return out.to(out_dtype)
 
 
+def qkv_norm_rope_write(q, k, v, wq, wk, eps, positions, inv_freq, rot_dims, interleaved, rot_mag, k_cache, v_cache, loc):
+    head_norm_rope(k, wk, eps, positions, inv_freq, rot_dims, interleaved, 1.0, k.dtype, cache=k_cache, loc=loc, rot_mag=rot_mag)
+    head_norm_rope(v, torch.ones(v.shape[2], dtype=v.dtype), eps, positions, inv_freq, 0, interleaved, 1.0, v.dtype, cache=v_cache, loc=loc)
+    return head_norm_rope(q, wq, eps, positions, inv_freq, rot_dims, interleaved, 1.0, q.dtype, rot_mag=rot_mag)
+
+
 def linear_recurrence(q, k, v, out, state, req_to_state, req_pool_indices, positions, q_scale, gate_logits=None, gate_bias=None,
-                      tau=1.0, head_decay=None, tok_req=None, seg_start=None, seg_len=None):
-    T, H, dk = q.shape
+                      tau=1.0, head_decay=None, tok_req=None, seg_start=None, seg_len=None, dt_logits=None, dt_bias=None,
+                      rate_log=None, skip=None):
+    T, G, dk = q.shape
+    H = v.shape[1]
+    rep = H // G
     S = None
     for t, (b, first, last) in enumerate(_segments(T, tok_req, seg_start, seg_len)):
         slot = int(req_to_state[int(req_pool_indices[b])])
         if first:
             S = torch.zeros_like(state[slot]) if int(positions[t]) == 0 else state[slot].clone()
-        if gate_logits is not None:
+        kk = k[t].float().repeat_interleave(rep, 0)
+        if dt_logits is not None:
+            dt = torch.nn.functional.softplus(dt_logits[t].float() + dt_bias.float())
+            a = torch.exp(-torch.exp(rate_log.float()) * dt)[:, None].expand(H, dk)
+            kk = kk * dt[:, None]
+        elif gate_logits is not None:
             z = gate_logits[t].float() + (gate_bias.float() if gate_bias is not None else 0.0)
             a = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(H, dk)
         else:
             a = head_decay.float()[:, None].expand(H, dk)
-        S = a[:, :, None] * S + k[t].float()[:, :, None] * v[t].float()[:, None, :]
-        out[t] = torch.einsum("hkv,hk->hv", S, q[t].float() * q_scale)
+        S = a[:, :, None] * S + kk[:, :, None] * v[t].float()[:, None, :]
+        out[t] = torch.einsum("hkv,hk->hv", S, q[t].float().repeat_interleave(rep, 0) * q_scale)
+        if skip is not None:
+            out[t] += skip.float()[:, None] * v[t].float()
         if last:
             state[slot] = S
     return out
@@ -545,7 +572,7 @@ def _act(z, act):
 
 
 def causal_conv(u, w1, state, req_to_state, req_pool_indices, positions, w2=None, residual=False, act="none", tok_req=None,
-                seg_start=None, seg_len=None):
+                seg_start=None, seg_len=None, bias=None):
     T, C = u.shape
     taps = w1.shape[1]
     outs = [torch.empty((T, C), dtype=u.dtype) for _ in range(1 if w2 is None else 2)]
@@ -562,6 +589,8 @@ def causal_conv(u, w1, state, req_to_state, req_pool_indices, positions, w2=None
                 acc = acc + w[:, taps - 1 - k].float() * hist[len(hist) - 1 - k]
             if residual:
                 acc = acc + hist[-1]
+            if bias is not None and w is w1:
+                acc = acc + bias.float()
             y[t] = _act(acc, act).to(u.dtype)
         hist = hist[1:]
         if last and taps > 1:
@@ -583,7 +612,9 @@ def gated_delta_rule(q, k, v, beta_logits, gate_logits, rate_bias, rate_log, out
         slot = int(req_to_state[int(req_pool_indices[b])])
         if first:
             S = torch.zeros_like(state[slot]) if int(positions[t]) == 0 else state[slot].clone()
-        a = torch.exp(-torch.exp(rate_log.float())[:, None] * F.softplus(gate_logits[t].float() + rate_bias.float()).view(H, dk))
+        z = F.softplus(gate_logits[t].float() + rate_bias.float())
+        z = z[:, None].expand(H, dk) if (gate_logits.shape[1] == H and rate_bias.numel() == H) else z.view(H, dk)
+        a = torch.exp(-torch.exp(rate_log.float())[:, None] * z)
         beta = torch.sigmoid(beta_logits[t].float())
         kk = k[t].float().repeat_interleave(rep, 0)
         qq = q[t].float().repeat_interleave(rep, 0) * q_scale
@@ -600,12 +631,24 @@ def window_attention_block_tokens(heads, kv_heads, head_dim, v_head_dim, dtype):
     return 3
 
 
-def window_attention_splits(tokens, heads, kv_heads, max_len, window, dtype):
+def window_attention_splits(tokens, heads, kv_heads, max_len, window, dtype, pool=0):
     return 1
 
 
+def pool_kv_blocks(k_cache, v_cache, pooled_k, pooled_v, req_to_token, req_pool_indices, positions, pool, pool_div=1, tok_req=None):
+    for t in range(positions.numel()):
+        pos = int(positions[t])
+        if (pos + 1) % pool:
+            continue
+        b = t if tok_req is None else int(tok_req[t])
+        slots = req_to_token[int(req_pool_indices[b]), pos - pool + 1: pos + 1].long()
+        dst = int(slots[-1]) // pool_div
+        pooled_k[dst] = (k_cache[slots].float().sum(0) / pool).to(pooled_k.dtype)
+        pooled_v[dst] = (v_cache[slots].float().sum(0) / pool).to(pooled_v.dtype)
+
+
 def window_attention(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, sink, window, scale, tok_req=None,
-                     blocks=None, max_run=None, num_splits=1):
+                     blocks=None, max_run=None, num_splits=1, pool=0, pooled_k=None, pooled_v=None, pool_div=1, head_gate=None):
     T, H, d = q.shape
     G = k_cache.shape[1]
     covered = torch.zeros(T, dtype=torch.bool)
@@ -620,13 +663,21 @@ def window_attention(q, k_cache, v_cache, out, req_to_token, req_pool_indices, p
             lo = max(0, pos - window + 1) if window > 0 else 0
             slots = req_to_token[int(req_pool_indices[b]), lo: pos + 1].long()
             kk, vv = k_cache[slots].float(), v_cache[slots].float()
+            if pool > 0 and window > 0:
+                seen = [bb for bb in range((pos + 1) // pool) if bb * pool + pool - 1 <= pos - window]
+                if seen:
+                    ends = req_to_token[int(req_pool_indices[b]), [bb * pool + pool - 1 for bb in seen]].long() // pool_div
+                    kk, vv = torch.cat([pooled_k[ends].float(), kk]), torch.cat([pooled_v[ends].float(), vv])
             for h in range(H):
                 g = h // (H // G)
                 s = (kk[:, g] @ q[t, h].float()) * scale
                 if sink is not None:
                     s = torch.cat([s, sink[h].float().reshape(1)])
-                p = torch.softmax(s, 0)[: slots.numel()]
-                out[t, h] = (p @ vv[:, g]).to(out.dtype)
+                p = torch.softmax(s, 0)[: kk.shape[0]]
+                o = p @ vv[:, g]
+                if head_gate is not None:
+                    o = o * torch.sigmoid(head_gate[t, h].float())
+                out[t, h] = o.to(out.dtype)
     assert bool(covered.all()), "the runs do not cover every token"
     return out
 
