@@ -46,6 +46,8 @@ FAMILY_SOURCES = {
                 "attn_sigmoid.hip", "moe_ops.hip"],
     "Gatarax": ["elementwise.hip", "index_ops.hip", "gemm.hip", "gemm_tiled.hip", "postnorm_ops.hip", "recurrence.hip",
                 "moe_ops.hip", "conv_ops.hip", "attn_window.hip"],
+    "Fudonex": ["elementwise.hip", "index_ops.hip", "gemm.hip", "gemm_tiled.hip", "postnorm_ops.hip", "recurrence.hip",
+                "conv_ops.hip", "attn_window.hip"],
 }
 PARTIAL_MARK = LIB + ".partial"
 

@@ -29,6 +29,9 @@ class ModelConfig:
         if self.architecture == "Gatarax":
             self._init_gatarax(c, dtype, context_length, quantization)
             return
+        if self.architecture == "Fudonex":
+            self._init_fudonex(c, dtype, context_length, quantization)
+            return
         self.hidden_size = c["hidden_size"]
         self.num_hidden_layers = c["num_hidden_layers"]
         self.num_attention_heads = c["num_attention_heads"]
@@ -202,6 +205,91 @@ class ModelConfig:
         self.recurrent_layer_shapes = [(s["mixer"]["right"]["heads"], s["mixer"]["right"]["dim"], s["mixer"]["right"]["vdim"])
                                        if s["type"] == "parallel" else (s["mixer"]["heads"], s["mixer"]["dim"], s["mixer"]["vdim"])
                                        for s in layers]
+
+    def _init_fudonex(self, c: dict, dtype: str, context_length: Optional[int], quantization: Optional[str]) -> None:
+        """The Fudonex design: "layers" lists the layers one by one, {"type": "attention" | "mamba2" | "delta", "mixer":
+        {...}, "mlp": {"kind": "dense", "ff"} | null}; widths under "width" / "vocab", the norms' epsilon under "norm", the
+        embedding's factor under "embedding", the factor on every sublayer's normed output under "residual_mult", the
+        cap of the logits under "logit_softcap".  An "attention" mixer keeps keys and values per token (kv_layer_shapes)
+        and, with "mask" {"size", "pool"}, averaged blocks of them (kv_layer_pools: the block lengths asked for by the
+        layer itself and by the layers that read its cache); with "kv_from": j it keeps none and reads layer j's
+        (kv_layer_sources), under a mask of its own.  "mamba2" and "delta" mixers keep one matrix per head and sequence
+        (recurrent_layer_shapes).  Layers may differ in every size."""
+        layers = c["layers"]
+        for i, spec in enumerate(layers):
+            if spec["type"] not in ("attention", "mamba2", "delta"):
+                raise ValueError(f"Fudonex layer {i}: unknown mixer type {spec['type']!r}")
+            if spec.get("mlp") is not None and spec["mlp"].get("kind") != "dense":
+                raise ValueError(f"Fudonex layer {i}: unknown feed-forward kind {spec['mlp'].get('kind')!r}")
+            m = spec["mixer"]
+            if spec["type"] == "attention":
+                if m["heads"] % m.get("kv_heads", m["heads"]):
+                    raise ValueError(f"Fudonex layer {i}: {m['heads']} query heads over {m['kv_heads']} key heads")
+                src = m.get("kv_from")
+                if src is not None:
+                    if not (0 <= src < i) or layers[src]["type"] != "attention" or layers[src]["mixer"].get("kv_from") is not None:
+                        raise ValueError(f"Fudonex layer {i}: kv_from {src} is not an earlier attention layer with keys of its own")
+                    s = layers[src]["mixer"]
+
+                    def kv_shape(x):
+                        return (x.get("kv_heads", x["heads"]), x["dim"], x.get("vdim", x["dim"]))
+
+                    if kv_shape(s) != kv_shape(m):
+                        raise ValueError(f"Fudonex layer {i}: its key / value shapes differ from layer {src}'s")
+                rot = m.get("rot")
+                if rot and (rot["dims"] % 2 or rot["dims"] > m["dim"]):
+                    raise ValueError(f"Fudonex layer {i}: rotation over {rot['dims']} of {m['dim']} features")
+            elif spec["type"] == "mamba2":
+                if m["heads"] % m.get("groups", 1) or (m["heads"] * m["vdim"]) % m.get("norm_groups", 1):
+                    raise ValueError(f"Fudonex layer {i}: heads, groups and norm groups do not divide")
+            elif m["heads"] % m.get("kv_heads", m["heads"]):
+                raise ValueError(f"Fudonex layer {i}: {m['heads']} heads over {m['kv_heads']} key heads")
+        self.layer_specs = layers
+        self.hidden_size = c["width"]
+        self.vocab_size = c["vocab"]
+        self.num_hidden_layers = len(layers)
+        att = [s["mixer"] for s in layers if s["type"] == "attention"]
+        self.num_attention_heads = max([m["heads"] for m in att] or [1])
+        self.num_key_value_heads = max([m.get("kv_heads", m["heads"]) for m in att] or [1])
+        self.head_dim = max([m["dim"] for m in att] or [1])
+        self.v_head_dim = max([m.get("vdim", m["dim"]) for m in att] or [1])
+        self.intermediate_size = max([s["mlp"]["ff"] for s in layers if s.get("mlp")] or [0])
+        self.rms_norm_eps = c["norm"]["eps"]
+        self.embedding_scale = float((c.get("embedding") or {}).get("scale", 1.0))
+        self.residual_mult = float(c.get("residual_mult", 1.0))
+        cap = c.get("logit_softcap")
+        self.final_logit_softcapping = float(cap) if cap else None
+        self.rope_theta = None
+        self.rope_scaling = None
+        self.tie_word_embeddings = True
+        self.max_position_embeddings = context_length or 131072     # the design fixes no longest sequence
+        self.context_len = self.max_position_embeddings
+        self.quantization = quantization
+        self.dtype = _DTYPES.get(dtype) or torch.bfloat16
+        self.is_encoder_decoder = False
+        self.needs_sequence_state = any(s["type"] != "attention" for s in layers)
+
+        def own_kv(s):
+            return s["type"] == "attention" and s["mixer"].get("kv_from") is None
+
+        self.kv_layer_shapes = [(s["mixer"].get("kv_heads", s["mixer"]["heads"]), s["mixer"]["dim"], s["mixer"].get("vdim", s["mixer"]["dim"]))
+                                if own_kv(s) else None for s in layers]
+        self.kv_layer_sources = {i: int(s["mixer"]["kv_from"]) for i, s in enumerate(layers)
+                                 if s["type"] == "attention" and s["mixer"].get("kv_from") is not None}
+        # the block lengths of a layer's averaged keys and values: its own mask's and those of the layers that read its cache
+        # (a reader has its own mask), so a tuple per owning layer
+        pools = []
+        for i, s in enumerate(layers):
+            sizes = set()
+            if own_kv(s):
+                readers = [s["mixer"]] + [layers[j]["mixer"] for j, src in self.kv_layer_sources.items() if src == i]
+                sizes = {int((r.get("mask") or {}).get("pool", 0) or 0) for r in readers if (r.get("mask") or {}).get("size", 0) > 0}
+                sizes.discard(0)
+            pools.append(tuple(sorted(sizes)))
+        self.kv_layer_pools = pools
+        self.recurrent_layer_shapes = [None if s["type"] == "attention" else
+                                       (s["mixer"]["heads"], s["mixer"]["state"] if s["type"] == "mamba2" else s["mixer"]["dim"],
+                                        s["mixer"]["vdim"]) for s in layers]
 
     @classmethod
     def from_path(cls, model_path: str, **kw) -> "ModelConfig":

@@ -333,24 +333,42 @@ class Mi355AttnBackend(AttentionBackend):
             tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq), num_splits=splits, max_run=bq)
 
     # ---- softmax attention over a sliding window with a sink term, per-layer key / value buffers ----
-    def forward_window(self, q, layer, forward_batch, out):
+    def store_window_blocks(self, layer, forward_batch):
+        """The averaged key / value row of every block that this step completes, for each block length in layer.store_pools."""
+        pool = forward_batch.token_to_kv_pool
+        k_cache, v_cache = pool.get_kv_buffer(layer.kv_layer_id)
+        for block in layer.store_pools:
+            pk, pv, div = pool.get_pooled_buffer(layer.kv_layer_id, block)
+            get_ops().pool_kv_blocks(k_cache, v_cache, pk, pv, forward_batch.req_to_token_pool.req_to_token, forward_batch.req_pool_indices,
+                                     forward_batch.positions, block, div, tok_req=forward_batch.token_req_index())
+
+    def forward_window(self, q, layer, forward_batch, out, head_gate=None):
         """q [T, H, d] -> out [T, H, dv]: softmax over the keys within layer.window positions, exp(sink_h) added to the
         denominator.  The new tokens' keys and values are in the cache already; prefill portions, decode steps and mixed
         batches are the same launch, told apart only by the list of token runs.  A decode step with few sequences cuts each
         token's visible keys into ranges that a second launch merges."""
         ops = get_ops()
-        k_cache, v_cache = forward_batch.token_to_kv_pool.get_kv_buffer(layer.layer_id)
+        kv_layer = getattr(layer, "kv_layer_id", layer.layer_id)
+        k_cache, v_cache = forward_batch.token_to_kv_pool.get_kv_buffer(kv_layer)
+        extra = {}
+        if getattr(layer, "pool", 0) > 0:
+            pk, pv, div = forward_batch.token_to_kv_pool.get_pooled_buffer(kv_layer, layer.pool)
+            extra = dict(pool=layer.pool, pooled_k=pk, pooled_v=pv, pool_div=div)
+        if head_gate is not None:
+            extra["head_gate"] = head_gate
         bq = ops.window_attention_block_tokens(layer.tp_q_head_num, layer.tp_k_head_num, layer.qk_head_dim, layer.v_head_dim, q.dtype)
         if q.stride(0) % 8 or q.stride(1) % 8:
             q = q.contiguous()      # a column block of a wider row that does not start every head on 16 bytes
         splits = 1
         if forward_batch.forward_mode.is_decode() and forward_batch.seq_lens_cpu is not None:
             splits = ops.window_attention_splits(q.shape[0], layer.tp_q_head_num, layer.tp_k_head_num,
-                                                 int(forward_batch.seq_lens_cpu.max()), layer.window, q.dtype)
+                                                 int(forward_batch.seq_lens_cpu.max()), layer.window, q.dtype,
+                                                 **({"pool": layer.pool} if extra.get("pool") else {}))
         return ops.window_attention(
             q, k_cache, v_cache, out, forward_batch.req_to_token_pool.req_to_token, forward_batch.req_pool_indices,
             forward_batch.positions, layer.sink.data if layer.sink is not None else None, layer.window, layer.scaling,
-            tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq), max_run=bq, num_splits=splits)
+            tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq), max_run=bq, num_splits=splits,
+            **extra)
 
     def _windowed(self, layer) -> bool:
         """triton_backend.py:656, 711: a layer with sliding_window_size > -1 attends the window lists."""

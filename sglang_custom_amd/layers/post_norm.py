@@ -5,7 +5,8 @@ reference, whose models norm before their sublayers and keep the residual in the
                       each divided by its own sqrt(mean(part^2) + eps).  The branch is a [T, D] tensor or a weighted sum
                       of rows of a larger tensor (the chosen experts' outputs of a mixture).  One launch, which also
                       writes the activation-dtype copy of the new x that the next projections read.
-  NormedResidualAdd   x <- x + y / sqrt(mean(y^2) + eps) * w in place, same second output.
+  NormedResidualAdd   x <- x + mult * ls * y / sqrt(mean(y^2) + eps) * (offset + w) in place, same second output: a norm on a
+                      sublayer's OUTPUT; offset 1 for a weight stored around zero, ls an optional per-channel layer scale.
 
 groups, eps and c are constructor arguments; all arithmetic is fp32 whatever the activation dtype."""
 from typing import Optional
@@ -36,10 +37,14 @@ class GroupRMSNorm(nn.Module):
 
 
 class NormedResidualAdd(nn.Module):
-    def __init__(self, hidden: int, eps: float, dtype, device):
+    def __init__(self, hidden: int, eps: float, dtype, device, offset: float = 0.0, mult: float = 1.0, layer_scale: bool = False):
         super().__init__()
-        self.eps = float(eps)
-        self.weight = nn.Parameter(torch.ones(hidden, dtype=dtype, device=device), requires_grad=False)
+        self.eps, self.offset, self.mult = float(eps), float(offset), float(mult)
+        self.weight = nn.Parameter((torch.zeros if offset else torch.ones)(hidden, dtype=dtype, device=device), requires_grad=False)
+        self.layer_scale = nn.Parameter(torch.ones(hidden, dtype=dtype, device=device), requires_grad=False) if layer_scale else None
 
     def forward(self, x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
-        return get_ops().rmsnorm_residual_add(x, y, self.weight.data, self.eps)
+        if self.offset == 0.0 and self.mult == 1.0 and self.layer_scale is None:
+            return get_ops().rmsnorm_residual_add(x, y, self.weight.data, self.eps)
+        return get_ops().rmsnorm_residual_add(x, y, self.weight.data, self.eps, offset=self.offset, mult=self.mult,
+                                              layer_scale=self.layer_scale.data if self.layer_scale is not None else None)

@@ -190,6 +190,32 @@ def rotate_half_inv_freq(base: float, dims: int) -> torch.Tensor:
     return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / max(dims, 1)).to(torch.float32)
 
 
+def scaled_pair_inv_freq(base: float, dims: int, scaling: Optional[dict]):
+    """Frequencies of a rotation over `dims` features stretched for sequences longer than the `original` length
+    (scaling = {"factor", "original", "fast", "slow"}; None: plain), and the magnitude that goes on cos and sin.  With
+    p(t) = dims ln(original / (2 pi t)) / (2 ln base) the index of the pair that turns t times over `original` positions,
+    lo = max(floor(p(fast)), 0), hi = min(ceil(p(slow)), dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1):
+    f'_i = f_i / factor * ramp_i + f_i (1 - ramp_i), magnitude 0.1 ln(factor) + 1.  The same interpolation as
+    yarn_inverse_frequencies; computed in float64 and rounded once, and with the span's lower bound as stated."""
+    half = dims // 2
+    f = [float(base) ** (-2.0 * i / dims) for i in range(half)]
+    if not scaling:
+        return torch.tensor(f, dtype=torch.float64).to(torch.float32), 1.0
+    factor, original = float(scaling["factor"]), float(scaling["original"])
+
+    def pair_index_for(turns: float) -> float:
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+    lo = max(math.floor(pair_index_for(float(scaling["fast"]))), 0)
+    hi = min(math.ceil(pair_index_for(float(scaling["slow"]))), dims - 1)
+    span = max(hi - lo, 0.001)
+    out = []
+    for i in range(half):
+        ramp = min(max((i - lo) / span, 0.0), 1.0)
+        out.append(f[i] / factor * ramp + f[i] * (1.0 - ramp))
+    return torch.tensor(out, dtype=torch.float64).to(torch.float32), 0.1 * math.log(factor) + 1.0
+
+
 def pair_inv_freq(base: float, dims: int) -> torch.Tensor:
     """The same frequencies for a rotation in either pairing (feature 2 i with 2 i + 1, or i with i + dims / 2): which
     features form pair i is the kernel's business, f_i is not."""

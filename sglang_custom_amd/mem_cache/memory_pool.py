@@ -277,9 +277,16 @@ class LayeredMHATokenToKVPool:
     """Keys and values per token for models whose layers differ: layer l has its own [size + page_size, heads_l, d_l]
     key buffer and [size + page_size, heads_l, dv_l] value buffer, or none at all (shapes[l] is None: a layer that
     keeps no keys, e.g. one with a recurrent mixer).  Slot 0 is the sink row of padded tokens, as in the other
-    pools; one slot index serves every layer."""
+    pools; one slot index serves every layer.
 
-    def __init__(self, size: int, page_size: int, dtype: torch.dtype, shapes: List[Optional[Tuple[int, int, int]]], device: str):
+    shared {layer: source layer}: the layer has no buffers of its own and reads (never writes) the source layer's.
+    pooled [layer] = (P, ...): for each block length P the layer also keeps one averaged key and value row per block of P
+    consecutive positions of a sequence, at row slot(block's last position) // div.  When pages are whole multiples of P slots a block's slots are
+    consecutive and aligned, so div = P and the pooled buffers hold rows / P rows; otherwise (single-slot pages, or a page
+    size that P does not divide) div = 1 and they are as long as the token buffers, sparsely used."""
+
+    def __init__(self, size: int, page_size: int, dtype: torch.dtype, shapes: List[Optional[Tuple[int, int, int]]], device: str,
+                 shared: Optional[dict] = None, pooled: Optional[List[Optional[Tuple[int, ...]]]] = None):
         self.size = size
         self.page_size = page_size
         self.dtype = dtype
@@ -290,15 +297,31 @@ class LayeredMHATokenToKVPool:
         rows = size + page_size
         self.k_buffer = [None if s is None else torch.zeros((rows, s[0], s[1]), dtype=dtype, device=device) for s in shapes]
         self.v_buffer = [None if s is None else torch.zeros((rows, s[0], s[2]), dtype=dtype, device=device) for s in shapes]
+        self.pooled = {}
+        for l, sizes in enumerate(pooled or []):
+            for p in (sizes or ()) if shapes[l] is not None else ():
+                div = p if page_size % p == 0 else 1
+                n = (rows + div - 1) // div
+                s = shapes[l]
+                self.pooled[(l, p)] = (torch.zeros((n, s[0], s[1]), dtype=dtype, device=device),
+                                       torch.zeros((n, s[0], s[2]), dtype=dtype, device=device), div)
+        self.shared = dict(shared or {})
+        for l, src in self.shared.items():
+            assert shapes[l] is None and self.k_buffer[src] is not None, f"layer {l} reads the cache of layer {src}, which has none"
 
     def get_kv_size_bytes(self) -> int:
-        return sum(b.numel() * b.element_size() for b in self.k_buffer + self.v_buffer if b is not None)
+        own = sum(b.numel() * b.element_size() for b in self.k_buffer + self.v_buffer if b is not None)
+        return own + sum(k.numel() * k.element_size() + v.numel() * v.element_size() for k, v, _ in self.pooled.values())
+
+    def get_pooled_buffer(self, layer_id: int, block: int):
+        """(averaged keys, averaged values, div) over blocks of `block` positions of the layer whose cache layer_id reads."""
+        return self.pooled[(self.shared.get(layer_id, layer_id), block)]
 
     def get_key_buffer(self, layer_id: int) -> torch.Tensor:
-        return self.k_buffer[layer_id]
+        return self.k_buffer[self.shared.get(layer_id, layer_id)]
 
     def get_value_buffer(self, layer_id: int) -> torch.Tensor:
-        return self.v_buffer[layer_id]
+        return self.v_buffer[self.shared.get(layer_id, layer_id)]
 
     def get_kv_buffer(self, layer_id: int):
-        return self.k_buffer[layer_id], self.v_buffer[layer_id]
+        return self.get_key_buffer(layer_id), self.get_value_buffer(layer_id)

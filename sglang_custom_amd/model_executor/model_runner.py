@@ -124,6 +124,11 @@ class ModelRunner:
         layered = getattr(cfg, "kv_layer_shapes", None)   # per-layer (kv heads, key width, value width) or None per layer
         if layered is not None:
             cell = max(1, sum(h * (dk + dv) for h, dk, dv in filter(None, layered))) * torch.finfo(self.kv_cache_dtype).bits // 8
+            # averaged blocks (kv_layer_pools): one more row per block of P slots, or per slot where pages do not hold whole blocks
+            page_ = max(1, int(getattr(sa, "page_size", 1) or 1))
+            for s, sizes in zip(layered, getattr(cfg, "kv_layer_pools", None) or []):
+                for p in (sizes or ()) if s is not None else ():
+                    cell += -(-s[0] * (s[1] + s[2]) * (torch.finfo(self.kv_cache_dtype).bits // 8) // (p if page_ % p == 0 else 1))
         elif latent is not None:
             cell = sum(r + d for r, d in latent) * torch.finfo(self.kv_cache_dtype).bits // 8
         elif mla:
@@ -150,7 +155,9 @@ class ModelRunner:
         if layered is not None:
             if self.kv_cache_dtype != self.dtype:
                 raise ValueError("a cache with per-layer shapes is stored in the model dtype")
-            self.token_to_kv_pool = LayeredMHATokenToKVPool(self.max_total_num_tokens, page, self.kv_cache_dtype, layered, self.device)
+            self.token_to_kv_pool = LayeredMHATokenToKVPool(self.max_total_num_tokens, page, self.kv_cache_dtype, layered, self.device,
+                                                            shared=getattr(cfg, "kv_layer_sources", None),
+                                                            pooled=getattr(cfg, "kv_layer_pools", None))
         elif latent is not None:
             if self.kv_cache_dtype != self.dtype:
                 raise ValueError("a latent cache with per-layer widths is stored in the model dtype")

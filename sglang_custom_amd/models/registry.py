@@ -1,6 +1,6 @@
 """Model classes by the architecture name a configuration gives (the role of the reference's ModelRegistry,
 python/sglang/srt/models/registry.py, reduced to the families this package has).  HuggingFace configurations name
-theirs under "architectures"; Seturax, Verozen and Gatarax configurations under "architecture"."""
+theirs under "architectures"; Seturax, Verozen, Gatarax and Fudonex configurations under "architecture"."""
 import importlib
 
 _ARCHITECTURES = {
@@ -10,6 +10,7 @@ _ARCHITECTURES = {
     "Seturax": ("seturax", "SeturaxForCausalLM"),
     "Verozen": ("verozen", "VerozenForCausalLM"),
     "Gatarax": ("gatarax", "GataraxForCausalLM"),
+    "Fudonex": ("fudonex", "FudonexForCausalLM"),
 }
 
 
