@@ -76,7 +76,8 @@ def parse_args():
     ap.add_argument("--design-compare", default=None, metavar="SIZE",
                     help="instead of the headline workload: prefill and decode throughput of the Seturax design beside the "
                          "dense DeepSeek stack (w2048, w4096, tiny), of the Verozen design beside Llama (vz2048, vz4096, "
-                         "vztiny), or of the Gatarax design beside Verozen (gx2048, gx4096, gxtiny), at equal layer sizes with random weights, and their hot kernels alone against the HBM / "
+                         "vztiny), of the Gatarax design beside Verozen (gx2048, gx4096, gxtiny), or of the Fudonex design beside Gatarax (fx2048, "
+                         "fx4096, fxtiny), at equal layer sizes with random weights, and their hot kernels alone against the HBM / "
                          "matrix-core peaks; prints one JSON line (sglang_custom_amd/bench_designs.py)")
     ap.add_argument("--dry-run", action="store_true",
                     help="rendezvous rehearsal without a GPU: every rank joins a gloo group, meets at the "
@@ -315,7 +316,8 @@ def main():
         from sglang_custom_amd import bench_designs
 
         run = (bench_designs.run_verozen if args.design_compare in bench_designs.VEROZEN_SIZES else
-               bench_designs.run_gatarax if args.design_compare in bench_designs.GATARAX_SIZES else bench_designs.run)
+               bench_designs.run_gatarax if args.design_compare in bench_designs.GATARAX_SIZES else
+               bench_designs.run_fudonex if args.design_compare in bench_designs.FUDONEX_SIZES else bench_designs.run)
         print(json.dumps(run(args.design_compare, dtype=args.dtype, steps=args.steps)), flush=True)
         return
     if "WORLD_SIZE" not in os.environ and args.gpus > 1:

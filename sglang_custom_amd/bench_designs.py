@@ -609,3 +609,248 @@ def run_gatarax(size: str, dtype: str = "bfloat16", steps: int = 32, prefill_bs:
     out["stream_decode"] = gatarax_stream_kernels(s, decode_bs, decode_bs)
     out["stream_prefill"] = gatarax_stream_kernels(s, prefill_bs * prefill_len, prefill_bs)
     return out
+
+
+# ------------------------------------------------------------------------------------------------ Fudonex beside Gatarax
+# Fudonex is compared with the package's closest model, Gatarax (an fp32 residual stream, windowed softmax attention with a
+# sink over per-layer caches, a gated delta rule and a linear recurrence with a matrix per head and sequence, short causal
+# convolutions with state): same width, depth, vocabulary, attention heads and head widths, window, recurrent heads and
+# widths.  Both run dense feed-forwards here, of equal weight count (gated: three matrices of ff; ungated: two of 1.5 ff).
+FUDONEX_SIZES = {
+    "fx2048": dict(width=2048, heads=16, kv_heads=4, dim=128, rec_heads=16, rec_kv_heads=16, rec_dim=64, rec_vdim=128, groups=4, norm_groups=4,
+                   ff=5632, layers=4, vocab=32768, window=512, pool=64, conv=4, rot=64),
+    "fx4096": dict(width=4096, heads=32, kv_heads=8, dim=128, rec_heads=32, rec_kv_heads=32, rec_dim=64, rec_vdim=128, groups=8, norm_groups=8,
+                   ff=11264, layers=4, vocab=32768, window=512, pool=64, conv=4, rot=64),
+    "fxtiny": dict(width=320, heads=8, kv_heads=2, dim=64, rec_heads=4, rec_kv_heads=2, rec_dim=32, rec_vdim=64, groups=2, norm_groups=2,
+                   ff=512, layers=4, vocab=2048, window=64, pool=16, conv=3, rot=32),
+}
+
+
+def fudonex_config(s: dict) -> dict:
+    mlp = dict(kind="dense", ff=s["ff"])
+    att = dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5,
+               mask=dict(size=s["window"], pool=s["pool"]),
+               rot=dict(base=10000.0, dims=s["rot"], scaling=dict(factor=4.0, original=2048, fast=16.0, slow=2.0)))
+    order = [dict(type="attention", mixer=att, mlp=mlp),
+             dict(type="mamba2", mlp=mlp, mixer=dict(heads=s["rec_heads"], vdim=s["rec_vdim"], state=s["rec_dim"], groups=s["groups"],
+                                                     norm_groups=s["norm_groups"], conv=s["conv"])),
+             dict(type="delta", mlp=mlp, mixer=dict(heads=s["rec_heads"], kv_heads=s["rec_kv_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"],
+                                                    conv=s["conv"])),
+             dict(type="attention", mixer=dict(att, kv_from=0), mlp=mlp)]
+    return dict(architecture="Fudonex", vocab=s["vocab"], width=s["width"], norm=dict(eps=1e-6), embedding=dict(scale=1.0), residual_mult=0.5,
+                logit_softcap=30.0, layers=[order[i % 4] for i in range(s["layers"])])
+
+
+def gatarax_dense_config(s: dict) -> dict:
+    mlp = dict(kind="dense", ff=s["ff"] * 3 // 2)
+    par = dict(type="parallel", mlp=mlp,
+               mixer=dict(left=dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], conv=s["conv"], scale=s["dim"] ** -0.5,
+                                    mask=dict(size=s["window"])),
+                          right=dict(heads=s["rec_heads"], kv_heads=s["rec_kv_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"], conv=s["conv"],
+                                     decay_rank=64, gate_rank=64)))
+    lit = dict(type="lightning", mlp=mlp, mixer=dict(heads=s["rec_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"],
+                                                     decay=[0.9 + 0.0123 * (i % 8) for i in range(s["rec_heads"])]))
+    order = [par, lit, par, lit]
+    return dict(architecture="Gatarax", vocab=s["vocab"], width=s["width"], logit_scale=1.0, norm=dict(eps=1e-6), embedding=dict(scale=1.0),
+                canon=dict(taps=s["conv"]), layers=[order[i % 4] for i in range(s["layers"])])
+
+
+def fudonex_mixer_kernels(s: dict, bs: int, ctx: int, prefill_bs: int, prefill_len: int) -> dict:
+    """The token mixers' launches alone, bf16, each beside the closest model's like launch on the same shapes.  Attention:
+    the same kernel with and without averaged blocks and the head gate (decode: bytes = every visible key and value row
+    once per sequence, the window's and the blocks'; prefill: flops 2 (d + dv) per visible query-key or query-block pair and
+    head), and the launch that writes the averages.  Recurrences: the state-space form beside the recurrence with a fixed
+    decay per head, the delta rule with a decay per head beside the one with a decay per key channel (decode: the matrices'
+    bytes, read and written; prefill: fp32 vector flops, 6 / 10 per matrix element and token)."""
+    from . import ops
+
+    dev, dt = "cuda", torch.bfloat16
+    H, G, d, W, P = s["heads"], s["kv_heads"], s["dim"], s["window"], s["pool"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    res = {}
+    slots = bs * ctx + 8
+    kc = torch.randn(slots, G, d, device=dev, generator=g).to(dt)
+    vc = torch.randn(slots, G, d, device=dev, generator=g).to(dt)
+    pk, pv = torch.randn_like(kc), torch.randn_like(vc)
+    rtt = (torch.arange(bs * ctx, device=dev, dtype=torch.int32) + 1).view(bs, ctx)
+    rpi = torch.arange(bs, device=dev)
+    q = torch.randn(bs, H, d, device=dev, generator=g).to(dt)
+    gate = torch.randn(bs, H, device=dev, generator=g).to(dt)
+    o = torch.empty_like(q)
+    sink = torch.zeros(H, device=dev)
+    pos = torch.full((bs,), ctx - 1, device=dev, dtype=torch.int64)
+    nblk = max(0, (ctx - 1 - W + 1) // P)
+    sp = ops.window_attention_splits(bs, H, G, ctx, W, dt, pool=P)
+    t = _timed(lambda: ops.window_attention(q, kc, vc, o, rtt, rpi, pos, sink, W, d ** -0.5, num_splits=sp, pool=P, pooled_k=pk, pooled_v=pv,
+                                            head_gate=gate), 20)
+    b = bs * (min(ctx, W) + nblk) * G * d * 2 * 2
+    res["fudonex_decode_attention"] = dict(us=round(t * 1e6, 1), splits=sp, keys=min(ctx, W) + nblk, gbs=round(b / t / 1e9),
+                                           of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    sp2 = ops.window_attention_splits(bs, H, G, ctx, W, dt)
+    t = _timed(lambda: ops.window_attention(q, kc, vc, o, rtt, rpi, pos, sink, W, d ** -0.5, num_splits=sp2), 20)
+    b = bs * min(ctx, W) * G * d * 2 * 2
+    res["gatarax_decode_attention"] = dict(us=round(t * 1e6, 1), splits=sp2, keys=min(ctx, W), gbs=round(b / t / 1e9),
+                                           of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    posb = torch.full((bs,), (ctx // P) * P - 1, device=dev, dtype=torch.int64)       # every sequence completes a block
+    t = _timed(lambda: ops.pool_kv_blocks(kc, vc, pk, pv, rtt, rpi, posb, P), 20)
+    res["pool_kv_blocks_decode (every sequence ends a block)"] = dict(us=round(t * 1e6, 1), gbs=round(bs * (P + 1) * G * d * 2 * 2 / t / 1e9))
+    # ---- prefill attention
+    T = prefill_bs * prefill_len
+    kp = torch.randn(T + 8, G, d, device=dev, generator=g).to(dt)
+    vp = torch.randn(T + 8, G, d, device=dev, generator=g).to(dt)
+    pkp, pvp = torch.randn_like(kp), torch.randn_like(vp)
+    rtp = (torch.arange(T, device=dev, dtype=torch.int32) + 1).view(prefill_bs, prefill_len)
+    qp = torch.randn(T, H, d, device=dev, generator=g).to(dt)
+    gp = torch.randn(T, H, device=dev, generator=g).to(dt)
+    op = torch.empty_like(qp)
+    posp = torch.arange(prefill_len, device=dev).repeat(prefill_bs)
+    tok_req = torch.repeat_interleave(torch.arange(prefill_bs, device=dev, dtype=torch.int32), prefill_len)
+    rpp = torch.arange(prefill_bs, device=dev)
+    bq = ops.window_attention_block_tokens(H, G, d, d, dt)
+    assert prefill_len % bq == 0
+    starts = torch.arange(0, T, bq, dtype=torch.int32)
+    blocks = torch.stack([starts, torch.full_like(starts, bq)], 1).to(dev)
+    t = _timed(lambda: ops.window_attention(qp, kp, vp, op, rtp, rpp, posp, sink, W, d ** -0.5, tok_req=tok_req, blocks=blocks, max_run=bq, pool=P,
+                                            pooled_k=pkp, pooled_v=pvp, head_gate=gp), 3)
+    pairs = prefill_bs * sum(min(i + 1, W) + max(0, (i - W + 1) // P) for i in range(prefill_len))
+    fl = pairs * H * 2 * 2 * d
+    res["fudonex_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3))
+    t = _timed(lambda: ops.window_attention(qp, kp, vp, op, rtp, rpp, posp, sink, W, d ** -0.5, tok_req=tok_req, blocks=blocks, max_run=bq), 3)
+    pairs = prefill_bs * sum(min(i + 1, W) for i in range(prefill_len))
+    fl = pairs * H * 2 * 2 * d
+    res["gatarax_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3))
+    t = _timed(lambda: ops.pool_kv_blocks(kp, vp, pkp, pvp, rtp, rpp, posp, P, tok_req=tok_req), 5)
+    res["pool_kv_blocks_prefill"] = dict(us=round(t * 1e6, 1), gbs=round(T * (1 + 1.0 / P) * G * d * 2 * 2 / t / 1e9))
+    # ---- the recurrences
+    RH, RG, dk, dv, MG = s["rec_heads"], s["rec_kv_heads"], s["rec_dim"], s["rec_vdim"], s["groups"]
+    state = torch.zeros(bs + 1, RH, dk, dv, device=dev)
+    r2s = torch.arange(1, bs + 1, device=dev, dtype=torch.int32)
+    zeros_h = torch.zeros(RH, device=dev)
+    ones_h = torch.ones(RH, device=dev)
+    decay = torch.full((RH,), 0.97, device=dev)
+    rb_c = torch.zeros(RH * dk, device=dev)
+    ss = torch.arange(0, T, prefill_len, device=dev, dtype=torch.int32)
+    sl = torch.full((prefill_bs,), prefill_len, device=dev, dtype=torch.int32)
+    for n, seg, reps in ((bs, {}, 20), (T, dict(tok_req=tok_req, seg_start=ss, seg_len=sl), 3)):
+        rp_, ps_ = (rpi, torch.full((bs,), ctx, device=dev, dtype=torch.int64)) if not seg else (rpp, posp)
+        xs = torch.randn(n, RH, dv, device=dev, generator=g).to(dt)
+        Bm, Cm = (torch.randn(n, MG, dk, device=dev, generator=g).to(dt) * 0.1 for _ in range(2))
+        dtl = torch.randn(n, RH, device=dev, generator=g)
+        od = torch.empty(n, RH, dv, device=dev)
+        t = _timed(lambda: ops.linear_recurrence(Cm, Bm, xs, od, state, r2s, rp_, ps_, 1.0, dt_logits=dtl, dt_bias=zeros_h, rate_log=zeros_h,
+                                                 skip=ones_h, **seg), reps)
+        qg, kg = (torch.randn(n, RH, dk, device=dev, generator=g).to(dt) * 0.1 for _ in range(2))
+        t2 = _timed(lambda: ops.linear_recurrence(qg, kg, xs, od, state, r2s, rp_, ps_, 1.0, head_decay=decay, **seg), reps)
+        qd = torch.nn.functional.normalize(torch.randn(n, RG, dk, device=dev, generator=g), dim=-1)
+        kd = torch.nn.functional.normalize(torch.randn(n, RG, dk, device=dev, generator=g), dim=-1)
+        ba = torch.randn(n, 2 * RH, device=dev, generator=g)
+        t3 = _timed(lambda: ops.gated_delta_rule(qd, kd, xs, ba[:, :RH], ba[:, RH:], zeros_h, zeros_h, od, state, r2s, rp_, ps_, dk ** -0.5, **seg), reps)
+        be = torch.randn(n, RH, device=dev, generator=g).to(dt)
+        z = torch.randn(n, RH * dk, device=dev, generator=g)
+        t4 = _timed(lambda: ops.gated_delta_rule(qd, kd, xs, be, z, rb_c, zeros_h, od, state, r2s, rp_, ps_, dk ** -0.5, **seg), reps)
+        state.zero_()
+        if not seg:
+            b = bs * RH * dk * dv * 4 * 2
+            for name, tt in (("fudonex_state_space_decode", t), ("gatarax_lightning_decode", t2), ("fudonex_delta_rule_decode", t3),
+                             ("gatarax_delta_rule_decode", t4)):
+                res[name] = dict(us=round(tt * 1e6, 1), gbs=round(b / tt / 1e9), of_hbm_peak=round(b / tt / HBM_PEAK, 3))
+        else:
+            for name, tt, fl_ in (("fudonex_state_space_prefill", t, 6), ("gatarax_lightning_prefill", t2, 6), ("fudonex_delta_rule_prefill", t3, 10),
+                                  ("gatarax_delta_rule_prefill", t4, 10)):
+                res[name] = dict(ms=round(tt * 1e3, 3), vector_tflops=round(T * RH * dk * dv * fl_ / tt / 1e12, 2),
+                                 tokens_per_s_per_sequence=round(prefill_len / tt))
+    return res
+
+
+def fudonex_stream_kernels(s: dict, tokens: int, segments: int) -> dict:
+    """The elementwise launches by bytes moved (bf16 activations, fp32 stream), each beside the closest model's like launch."""
+    from . import ops
+    from .layers.rotary_embedding import pair_inv_freq, scaled_pair_inv_freq
+
+    dev, dt = "cuda", torch.bfloat16
+    D = s["width"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    res = {}
+    x = torch.randn(tokens, D, device=dev, generator=g)
+    y = torch.randn(tokens, D, device=dev, generator=g).to(dt)
+    w = torch.zeros(D, device=dev, dtype=dt)
+    ls = torch.ones(D, device=dev, dtype=dt)
+    t = _timed(lambda: ops.rmsnorm_residual_add(x, y, w, 1e-6, offset=1.0, layer_scale=ls, mult=0.5), 20)
+    res["rmsnorm_residual_add (offset weight, layer scale)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 4 + 2 + 2) / t / 1e9))
+    t = _timed(lambda: ops.branch_residual_add(x, y, ls, eps=1e-6), 20)
+    res["branch_residual_add, one normed branch (closest)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 4 + 2) / t / 1e9))
+    t = _timed(lambda: ops.offset_rmsnorm(x, w, 1e-6, 1.0), 20)
+    res["offset_rmsnorm (closest, the norm in front of a sublayer)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 2) / t / 1e9))
+    # gate, then group norm  |  head norm, then gate
+    RH, dv = s["rec_heads"], s["rec_vdim"]
+    inner = RH * dv
+    yv = torch.randn(tokens, inner, device=dev, generator=g)
+    z = torch.randn(tokens, inner, device=dev, generator=g).to(dt)
+    wi = torch.ones(inner, device=dev, dtype=dt)
+    t = _timed(lambda: ops.gated_group_rmsnorm(yv, z, wi, s["norm_groups"], 1e-6), 20)
+    res["gated_group_rmsnorm"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * inner * (4 + 2 + 2) / t / 1e9))
+    wv = torch.ones(dv, device=dev, dtype=dt)
+    t = _timed(lambda: ops.head_rmsnorm_gate_act(yv.view(tokens, RH, dv), wv, z, 1e-6, dt, "sigmoid"), 20)
+    res["head_rmsnorm_gate (closest)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * inner * (4 + 2 + 2) / t / 1e9))
+    # convolution over x | B | C with bias and silu  |  over q | k | v with silu
+    C = inner + 2 * s["groups"] * s["rec_dim"]
+    taps = s["conv"]
+    u = torch.randn(tokens, C + inner, device=dev, generator=g).to(dt)[:, inner:]
+    w1 = torch.randn(C, taps, device=dev, generator=g).to(dt)
+    bias = torch.randn(C, device=dev, generator=g).to(dt)
+    state = torch.zeros(segments + 1, taps - 1, C, device=dev)
+    r2s = torch.arange(1, segments + 1, device=dev, dtype=torch.int32)
+    rpi = torch.arange(segments, device=dev)
+    per = tokens // segments
+    if per == 1:
+        seg, pos = {}, torch.full((tokens,), 100, device=dev, dtype=torch.int64)
+    else:
+        seg = dict(tok_req=torch.repeat_interleave(torch.arange(segments, device=dev, dtype=torch.int32), per),
+                   seg_start=torch.arange(0, tokens, per, device=dev, dtype=torch.int32),
+                   seg_len=torch.full((segments,), per, device=dev, dtype=torch.int32))
+        pos = torch.arange(per, device=dev).repeat(segments)
+    t = _timed(lambda: ops.causal_conv(u, w1, state, r2s, rpi, pos, act="silu", bias=bias, **seg), 20)
+    res["causal_conv (bias, silu; with the state's update)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * C * 2 * 2 / t / 1e9))
+    t = _timed(lambda: ops.causal_conv(u, w1, state, r2s, rpi, pos, act="silu", **seg), 20)
+    res["causal_conv (silu; closest)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * C * 2 * 2 / t / 1e9))
+    # head norm + rotation of q (scaled frequencies and magnitude | plain)
+    H, d = s["heads"], s["dim"]
+    qs = torch.randn(tokens, H * d + 64, device=dev, generator=g).to(dt)[:, : H * d].view(tokens, H, d)
+    wq = torch.ones(d, device=dev, dtype=dt)
+    f, mag = scaled_pair_inv_freq(10000.0, s["rot"], dict(factor=4.0, original=2048, fast=16.0, slow=2.0))
+    f, f0 = f.to(dev), pair_inv_freq(10000.0, s["rot"]).to(dev)
+    t = _timed(lambda: ops.head_norm_rope(qs, wq, 1e-6, pos, f, s["rot"], False, 1.0, dt, rot_mag=mag), 20)
+    res["head_norm_rope (scaled frequencies, magnitude)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * H * d * 2 * 2 / t / 1e9))
+    t = _timed(lambda: ops.head_norm_rope(qs, wq, 1e-6, pos, f0, s["rot"], False, 1.0, dt), 20)
+    res["head_norm_rope (closest)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * H * d * 2 * 2 / t / 1e9))
+    # q, k and v of an attention layer: one launch beside the three it replaces
+    G = s["kv_heads"]
+    qkv = torch.randn(tokens, (H + 2 * G) * d + 64, device=dev, generator=g).to(dt)
+    q_, k_, v_ = qkv[:, : H * d].view(tokens, H, d), qkv[:, H * d: (H + G) * d].view(tokens, G, d), qkv[:, (H + G) * d: (H + 2 * G) * d].view(tokens, G, d)
+    kc, vc = torch.zeros(tokens + 8, G, d, device=dev, dtype=dt), torch.zeros(tokens + 8, G, d, device=dev, dtype=dt)
+    loc = torch.arange(1, tokens + 1, device=dev)
+    byt = tokens * (H + 2 * G) * d * 2 * 2
+    t = _timed(lambda: ops.qkv_norm_rope_write(q_, k_, v_, wq, wq, 1e-6, pos, f, s["rot"], False, mag, kc, vc, loc), 20)
+    res["qkv_norm_rope_write (one launch)"] = dict(us=round(t * 1e6, 1), gbs=round(byt / t / 1e9))
+
+    def three():
+        ops.head_norm_rope(q_, wq, 1e-6, pos, f, s["rot"], False, 1.0, dt, rot_mag=mag)
+        ops.head_norm_rope(k_, wq, 1e-6, pos, f, s["rot"], False, 1.0, dt, cache=kc, loc=loc, rot_mag=mag)
+        ops.head_norm_rope(v_, wq, 1e-6, pos, f, 0, False, 1.0, dt, cache=vc, loc=loc)
+    t = _timed(three, 20)
+    res["head_norm_rope x 3 (what it replaces)"] = dict(us=round(t * 1e6, 1), gbs=round(byt / t / 1e9))
+    return res
+
+
+def run_fudonex(size: str, dtype: str = "bfloat16", steps: int = 32, prefill_bs: int = 4, prefill_len: int = 2048, decode_bs: int = 64,
+                decode_ctx: int = 1024) -> dict:
+    s = FUDONEX_SIZES[size]
+    if size == "fxtiny":
+        prefill_bs, prefill_len, decode_bs, decode_ctx = 2, 256, 8, 128
+    out = dict(size=size, shape=s, dtype=dtype, data="synthetic", workload=dict(prefill=[prefill_bs, prefill_len], decode=[decode_bs, decode_ctx], steps=steps))
+    out["fudonex"] = model_throughput(fudonex_config(s), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=False)
+    out["gatarax"] = model_throughput(gatarax_dense_config(s), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=False)
+    out["mixers"] = fudonex_mixer_kernels(s, decode_bs, decode_ctx, prefill_bs, prefill_len)
+    out["stream_decode"] = fudonex_stream_kernels(s, decode_bs, decode_bs)
+    out["stream_prefill"] = fudonex_stream_kernels(s, prefill_bs * prefill_len, prefill_bs)
+    return out
